@@ -1,0 +1,162 @@
+"""ctypes view of include/nce_hip.h and include/nce_params.h, and the loader of libnce_hip.so.
+
+The shared library is the product: loading fails loudly when it has not been built, and nothing
+here falls back to a CPU implementation.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnce_hip.so")
+
+# nce_result_t
+SUCCESS = 0
+ERROR_OUT_OF_MEMORY = 0x70000002
+ERROR_INVALID_ARGUMENT = 0x78000004
+ERROR_INVALID_NULL_HANDLE = 0x78000005
+ERROR_UNSUPPORTED = 0x78000008
+ERROR_IO = 0x78000009
+ERROR_UNKNOWN = 0x7FFFFFFE
+RESULT_NAMES = {
+    SUCCESS: "NCE_RESULT_SUCCESS",
+    ERROR_OUT_OF_MEMORY: "NCE_RESULT_ERROR_OUT_OF_MEMORY",
+    ERROR_INVALID_ARGUMENT: "NCE_RESULT_ERROR_INVALID_ARGUMENT",
+    ERROR_INVALID_NULL_HANDLE: "NCE_RESULT_ERROR_INVALID_NULL_HANDLE",
+    ERROR_UNSUPPORTED: "NCE_RESULT_ERROR_UNSUPPORTED",
+    ERROR_IO: "NCE_RESULT_ERROR_IO",
+    ERROR_UNKNOWN: "NCE_RESULT_ERROR_UNKNOWN",
+}
+
+# nce_task_type_t = VPUIP::NCETaskType
+TASK_CONV, TASK_DWCONV, TASK_MAXPOOL, TASK_AVEPOOL, TASK_ELTWISE = 0, 1, 2, 3, 5
+# nce_ppe_mode_t = VPU::PPEMode
+PPE_NOOP, PPE_ADD, PPE_LRELU, PPE_LRELUX, PPE_LPRELU = 3, 5, 13, 14, 15
+# nce_mpe_mode_t = VPU::MPEMode
+MPE_VECTOR, MPE_MATRIX, MPE_VECTOR_FP16, MPE_CUBOID_16x16, MPE_CUBOID_8x16, MPE_CUBOID_4x16, MPE_NOP = range(7)
+# nce_dtype_t
+DT_U8, DT_I8, DT_SI32 = 0, 1, 2
+# nce_round_mode_t / nce_clamp_domain_t
+ROUND_HALF_UP, ROUND_HALF_EVEN, ROUND_NONE = 0, 1, 2
+CLAMP_POST_ZP, CLAMP_PRE_ZP = 0, 1
+# nce_arch_t / nce_postop_t (nce_params.h)
+ARCH_VPUX30XX, ARCH_VPUX37XX = 0, 1
+POSTOP_NONE, POSTOP_RELU, POSTOP_CLAMP, POSTOP_LEAKY_RELU = 0, 1, 2, 3
+
+INT32_MIN, INT32_MAX = -(2**31), 2**31 - 1
+
+
+class Tensor(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p),
+        ("dtype", C.c_int32),
+        ("zero_point", C.c_int32),
+        ("dims", C.c_int64 * 4),
+        ("strides_bytes", C.c_int64 * 4),
+    ]
+
+
+class DpuTask(C.Structure):
+    _fields_ = [
+        ("out_start", C.c_int32 * 3),
+        ("out_end", C.c_int32 * 3),
+        ("pad_left", C.c_int32),
+        ("pad_right", C.c_int32),
+        ("pad_top", C.c_int32),
+        ("pad_bottom", C.c_int32),
+        ("mpe_mode", C.c_int32),
+        ("cluster_id", C.c_int32),
+    ]
+
+
+class PpeTask(C.Structure):
+    _fields_ = [
+        ("mode", C.c_int32),
+        ("clamp_low", C.c_int32),
+        ("clamp_high", C.c_int32),
+        ("lrelu_mult", C.c_int32),
+        ("lrelu_shift", C.c_int32),
+        ("has_quant", C.c_int32),
+        ("quant_mult", C.c_int32),
+        ("quant_shift", C.c_int32),
+        ("quant_post_shift", C.c_int32),
+        ("has_in_mult", C.c_int32),
+        ("in1_quant_mult", C.c_int32),
+        ("in2_quant_mult", C.c_int32),
+        ("round_mode", C.c_int32),
+        ("clamp_domain", C.c_int32),
+    ]
+
+
+class ClusterTaskDesc(C.Structure):
+    _fields_ = [
+        ("task_type", C.c_int32),
+        ("flags", C.c_uint32),
+        ("input", Tensor),
+        ("weights", Tensor),
+        ("weight_table", Tensor),
+        ("output", Tensor),
+        ("kernel_size", C.c_int32 * 2),
+        ("kernel_strides", C.c_int32 * 2),
+        ("kernel_pad_left", C.c_int32),
+        ("kernel_pad_right", C.c_int32),
+        ("kernel_pad_top", C.c_int32),
+        ("kernel_pad_bottom", C.c_int32),
+        ("variants", C.POINTER(DpuTask)),
+        ("num_variants", C.c_uint32),
+        ("reserved", C.c_uint32),
+        ("ppe", C.POINTER(PpeTask)),
+    ]
+
+
+class ExecutorDesc(C.Structure):
+    _fields_ = [("device_id", C.c_int32), ("log_level", C.c_int32)]
+
+
+class Quant(C.Structure):
+    _fields_ = [("scale", C.c_double), ("zero_point", C.c_int32), ("dtype", C.c_int32)]
+
+
+# Every symbol the two headers declare: name -> (restype, argtypes)
+_P = C.POINTER
+SYMBOLS = {
+    "nceGetVersion": (C.c_int, [_P(C.c_uint32), _P(C.c_uint32)]),
+    "nceExecutorCreate": (C.c_int, [ExecutorDesc, _P(C.c_void_p), _P(C.c_void_p)]),
+    "nceExecutorDestroy": (C.c_int, [C.c_void_p]),
+    "nceClusterTaskValidate": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc)]),
+    "nceClusterTaskEnqueue": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc), C.c_void_p]),
+    "nceTaskListCreate": (C.c_int, [C.c_void_p, _P(C.c_void_p)]),
+    "nceTaskListAppend": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc)]),
+    "nceTaskListEnqueue": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "nceTaskListDestroy": (C.c_int, [C.c_void_p]),
+    "nceExecutorSynchronize": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "nceLogHandleGetString": (C.c_int, [C.c_void_p, _P(C.c_size_t), C.c_char_p]),
+    "nceQuantApproximate": (C.c_int, [C.c_int32, C.c_double, _P(C.c_int32), _P(C.c_int32), _P(C.c_int32)]),
+    "nceEltwiseQuantApproximate": (C.c_int, [C.c_int32, C.c_double, C.c_double, C.c_double] + [_P(C.c_int32)] * 4),
+    "ncePReLUApproximate": (C.c_int, [C.c_int32, C.c_double, _P(C.c_int32), _P(C.c_int32)]),
+    "nceWeightsTableFill": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_double, C.c_double,
+                                      _P(C.c_double), C.c_int32, _P(C.c_double), _P(C.c_int32)]),
+    "ncePpeFromPostOp": (C.c_int, [C.c_int32, C.c_int32, C.c_double, C.c_double, Quant, _P(PpeTask)]),
+    "ncePpeForAvgPool": (C.c_int, [C.c_int32, Quant, Quant, C.c_int32, C.c_int32, C.c_int32, C.c_double, C.c_double,
+                                   _P(PpeTask)]),
+    "ncePpeForEltwiseAdd": (C.c_int, [C.c_int32, Quant, Quant, Quant, C.c_int32, C.c_double, C.c_double, _P(PpeTask)]),
+}
+
+_lib = None
+
+
+def load_library():
+    """Load libnce_hip.so (built in-tree by `make -C npu_plugin_amd/csrc` or __graft_entry__.build())."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build the HIP library first (python -c 'import __graft_entry__ as g; g.build()'). "
+            "There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib

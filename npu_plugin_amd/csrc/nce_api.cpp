@@ -1,0 +1,541 @@
+// Host side of the C-ABI declared in include/nce_hip.h: handles, log, descriptor validation
+// (the rules of the reference's NCEClusterTaskOp verifier) and dispatch to the HIP kernels.
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "nce_common.h"
+
+struct nce_log_s {
+    std::mutex mu;
+    std::string text;
+    int level = 1;
+
+    void add(int lvl, const char* fmt, ...) {
+        if (lvl > level) return;
+        char buf[1024];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof(buf), fmt, ap);
+        va_end(ap);
+        std::lock_guard<std::mutex> lk(mu);
+        if (text.size() > (1u << 20)) text.clear();  // bounded
+        text += buf;
+        text += '\n';
+    }
+};
+
+struct nce_executor_s {
+    int device = 0;
+    nce_log_s* log = nullptr;
+};
+
+namespace {
+
+using nce::Box;
+using nce::PpeDev;
+using nce::TaskDev;
+using nce::TensorDev;
+
+constexpr int64_t kMaxKernel = 11;  // VPU::NCEInvariant::MAX_KERNEL_SIZE
+constexpr int64_t kMaxStride = 8;   // NCE_MAX_STRIDE_SIZE, src/vpux_compiler/src/dialect/VPUIP/nce_invariant.cpp:1062
+
+struct Plan {
+    TaskDev dev;
+    std::vector<Box> boxes;
+    int task_type = 0;
+};
+
+#define FAIL(code, ...)              \
+    do {                             \
+        log->add(1, __VA_ARGS__);    \
+        return code;                 \
+    } while (0)
+
+bool is_8bit(int32_t dt) {
+    return dt == NCE_DT_U8 || dt == NCE_DT_I8;
+}
+
+void type_range(int32_t dt, int64_t* lo, int64_t* hi) {
+    if (dt == NCE_DT_U8) {
+        *lo = 0;
+        *hi = 255;
+    } else {
+        *lo = -128;
+        *hi = 127;
+    }
+}
+
+int64_t clamp64(int64_t v, int64_t lo, int64_t hi) {
+    return v < lo ? lo : (v > hi ? hi : v);
+}
+
+// Activation tensor: NHWC, channels compact and a multiple of 16 for 8-bit types
+// (nce_cluster_task.cpp:346-359,702-709; src/vpux_compiler/src/dialect/VPU/utils/nce_invariant.cpp:135-153).
+nce_result_t check_activation(nce_log_s* log, const char* name, const nce_tensor_t& x, TensorDev* out) {
+    if (x.data == nullptr) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: data pointer is null", name);
+    if (!is_8bit(x.dtype)) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: only u8 / i8 storage is supported, got dtype %d", name, x.dtype);
+    for (int i = 0; i < 4; ++i)
+        if (x.dims[i] <= 0 || x.dims[i] > 0x7fffffff) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: dims[%d] = %lld", name, i, (long long)x.dims[i]);
+    if (x.dims[1] % 16 != 0) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: channels (%lld) must be a multiple of 16", name, (long long)x.dims[1]);
+    if (x.strides_bytes[1] != 1) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: layout must be NHWC with compact channels (C stride %lld)", name, (long long)x.strides_bytes[1]);
+    if (x.strides_bytes[3] < x.dims[1] || x.strides_bytes[2] < x.strides_bytes[3] * 1 || x.strides_bytes[0] < x.strides_bytes[2])
+        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides are not NHWC-ordered (N %lld, H %lld, W %lld, C 1)", name,
+             (long long)x.strides_bytes[0], (long long)x.strides_bytes[2], (long long)x.strides_bytes[3]);
+    if (((uintptr_t)x.data | (uintptr_t)x.strides_bytes[0] | (uintptr_t)x.strides_bytes[2] | (uintptr_t)x.strides_bytes[3]) & 15)
+        FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
+    int64_t lo, hi;
+    type_range(x.dtype, &lo, &hi);
+    if (x.zero_point < lo || x.zero_point > hi) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: zero point %d outside the storage range", name, x.zero_point);
+    out->data = static_cast<uint8_t*>(x.data);
+    out->sn = x.strides_bytes[0];
+    out->sh = x.strides_bytes[2];
+    out->sw = x.strides_bytes[3];
+    out->n = (int32_t)x.dims[0];
+    out->c = (int32_t)x.dims[1];
+    out->h = (int32_t)x.dims[2];
+    out->w = (int32_t)x.dims[3];
+    out->is_signed = x.dtype == NCE_DT_I8;
+    out->zp = x.zero_point;
+    return NCE_RESULT_SUCCESS;
+}
+
+// Weight table: [OC,1,1,4] si32, at least 4*OC elements (nce_cluster_task.cpp:361-416; shape
+// src/vpux_compiler/src/dialect/VPU/utils/nce_sparsity.cpp:633-635).
+nce_result_t check_table(nce_log_s* log, const nce_tensor_t& x, int64_t oc, TaskDev* dev) {
+    if (x.dtype != NCE_DT_SI32) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weight_table: element type must be si32");
+    int64_t elems = 1;
+    for (int i = 0; i < 4; ++i) {
+        if (x.dims[i] <= 0) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weight_table: dims[%d] = %lld", i, (long long)x.dims[i]);
+        elems *= x.dims[i];
+    }
+    if (elems < 4 * oc) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weight_table: %lld elements, need %lld (4 per output channel)", (long long)elems, (long long)(4 * oc));
+    if (x.strides_bytes[0] < 16 || x.strides_bytes[0] % 16 != 0 || ((uintptr_t)x.data & 15))
+        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weight_table: rows must be 16 bytes apart or more and 16-byte aligned");
+    dev->table = static_cast<const int32_t*>(x.data);
+    dev->table_stride = x.strides_bytes[0] / 4;
+    return NCE_RESULT_SUCCESS;
+}
+
+// verifyKernel, src/vpux_compiler/src/dialect/VPUIP/nce_invariant.cpp:1056-1108 (37XX: SX may differ from SY).
+nce_result_t check_kernel(nce_log_s* log, const nce_cluster_task_desc_t* t) {
+    const int64_t KY = t->kernel_size[0], KX = t->kernel_size[1], SY = t->kernel_strides[0], SX = t->kernel_strides[1];
+    if (KY <= 0 || KY > kMaxKernel) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "unsupported kernel height %lld, must be in [1, %lld]", (long long)KY, (long long)kMaxKernel);
+    if (KX <= 0 || KX > kMaxKernel) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "unsupported kernel width %lld, must be in [1, %lld]", (long long)KX, (long long)kMaxKernel);
+    if (SY <= 0 || SY > kMaxStride) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "unsupported stride height %lld, must be in [1, %lld]", (long long)SY, (long long)kMaxStride);
+    if (SX <= 0 || SX > kMaxStride) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "unsupported stride width %lld, must be in [1, %lld]", (long long)SX, (long long)kMaxStride);
+    const int64_t pads[4] = {t->kernel_pad_top, t->kernel_pad_bottom, t->kernel_pad_left, t->kernel_pad_right};
+    const int64_t lim[4] = {KY / 2, KY / 2, KX / 2, KX / 2};
+    for (int i = 0; i < 4; ++i)
+        if (pads[i] < 0 || (pads[i] > 1 && pads[i] > lim[i]))
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "unsupported padding %lld, must be in [0, %lld]", (long long)pads[i], (long long)std::max<int64_t>(1, lim[i]));
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t check_out_shape(nce_log_s* log, const nce_cluster_task_desc_t* t, const TensorDev& in, const TensorDev& out) {
+    const int64_t eh = ((int64_t)in.h + t->kernel_pad_top + t->kernel_pad_bottom - t->kernel_size[0]) / t->kernel_strides[0] + 1;
+    const int64_t ew = ((int64_t)in.w + t->kernel_pad_left + t->kernel_pad_right - t->kernel_size[1]) / t->kernel_strides[1] + 1;
+    if ((int64_t)in.h + t->kernel_pad_top + t->kernel_pad_bottom < t->kernel_size[0] ||
+        (int64_t)in.w + t->kernel_pad_left + t->kernel_pad_right < t->kernel_size[1])
+        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "kernel is larger than the padded input");
+    if (out.h != eh || out.w != ew)
+        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "output is %dx%d, kernel/stride/pad give %lldx%lld", out.h, out.w, (long long)eh, (long long)ew);
+    if (out.n != in.n) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "output batch %d differs from input batch %d", out.n, in.n);
+    return NCE_RESULT_SUCCESS;
+}
+
+// PPETask -> the form the kernels use. Mode handling follows setupQuantInQuantOut
+// (runtime_dpu_parser_imports.cpp.inc:511-542); limits of the PReLU registers:
+// src/vpux_compiler/src/dialect/VPU/transforms/passes/setup_ppe.cpp:77-92.
+nce_result_t build_ppe(nce_log_s* log, const nce_cluster_task_desc_t* t, const nce_tensor_t& out, bool has_table, PpeDev* d) {
+    static const nce_ppe_task_t kDefault = {NCE_PPE_NOOP, INT32_MIN, INT32_MAX, 1, 0, 0, 1, 0, 0, 0, 1, 1, NCE_ROUND_HALF_UP, NCE_CLAMP_POST_ZP};
+    const nce_ppe_task_t& p = t->ppe ? *t->ppe : kDefault;
+    d->prelu_mult = 1;
+    d->prelu_shift = 0;
+    switch (p.mode) {
+    case NCE_PPE_NOOP:
+    case NCE_PPE_ADD:
+        break;
+    case NCE_PPE_LRELU:
+    case NCE_PPE_LRELUX:
+        d->prelu_mult = 0;
+        break;
+    case NCE_PPE_LPRELU: {
+        const int64_t am = p.lrelu_mult < 0 ? -(int64_t)p.lrelu_mult : p.lrelu_mult;
+        if (am & ~(int64_t)0x7FF) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: ReLU multiplier %d exceeds 11 bits", p.lrelu_mult);
+        if (p.lrelu_shift & ~0x1F) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: ReLU shift %d does not fit 5 bits", p.lrelu_shift);
+        d->prelu_mult = p.lrelu_mult;
+        d->prelu_shift = p.lrelu_shift;
+        break;
+    }
+    default:
+        FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "ppe: mode %d is not part of the INT8 path", p.mode);
+    }
+    if (p.round_mode < NCE_ROUND_HALF_UP || p.round_mode > NCE_ROUND_NONE) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: round_mode %d", p.round_mode);
+    if (p.clamp_domain != NCE_CLAMP_POST_ZP && p.clamp_domain != NCE_CLAMP_PRE_ZP) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: clamp_domain %d", p.clamp_domain);
+    if (p.clamp_low > p.clamp_high) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: clamp_low %d > clamp_high %d", p.clamp_low, p.clamp_high);
+    d->round_mode = p.round_mode;
+
+    int64_t tlo, thi;
+    type_range(out.dtype, &tlo, &thi);
+    const bool is_max = t->task_type == NCE_TASK_MAXPOOL;
+    const int64_t zp = is_max ? 0 : out.zero_point;  // MAXPOOL: zero point register forced to 0 (…inc:2002-2004)
+    int64_t lo = p.clamp_low, hi = p.clamp_high;
+    if (p.clamp_domain == NCE_CLAMP_PRE_ZP && !is_max) {
+        lo += zp;
+        hi += zp;
+    }
+    d->lo = (int32_t)(clamp64(lo, tlo, thi) - zp);
+    d->hi = (int32_t)(clamp64(hi, tlo, thi) - zp);
+    d->zp_out = (int32_t)zp;
+
+    d->quant_mult = 1;
+    d->quant_shift = 0;
+    d->in1_mult = d->in2_mult = 1;
+    const bool needs_quant = (t->task_type == NCE_TASK_ELTWISE || t->task_type == NCE_TASK_AVEPOOL) && !has_table;
+    if (needs_quant) {
+        if (!p.has_quant) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: task has no weight table, so quant_mult / quant_shift are required");
+        if (p.quant_mult < 0 || p.quant_mult > 65535) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: quant_mult %d does not fit 16 bits", p.quant_mult);
+        if (p.quant_shift < 0 || p.quant_shift > 63) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: quant_shift %d does not fit 6 bits", p.quant_shift);
+        if (p.quant_post_shift != 0) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "ppe: quant_post_shift is a 30XX feature");
+        d->quant_mult = p.quant_mult;
+        d->quant_shift = p.quant_shift;
+    }
+    if (t->task_type == NCE_TASK_ELTWISE && p.has_in_mult) {
+        if (p.in1_quant_mult < 0 || p.in1_quant_mult > 65535 || p.in2_quant_mult < 0 || p.in2_quant_mult > 65535)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ppe: in1/in2_quant_mult must fit 16 bits");
+        d->in1_mult = p.in1_quant_mult;
+        d->in2_mult = p.in2_quant_mult;
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+int64_t box_volume(const Box& b) {
+    return (int64_t)b.bw * b.bh * b.bc;
+}
+
+bool boxes_overlap(const Box& a, const Box& b) {
+    return a.x0 < b.x0 + b.bw && b.x0 < a.x0 + a.bw && a.y0 < b.y0 + b.bh && b.y0 < a.y0 + a.bh && a.z0 < b.z0 + b.bc &&
+           b.z0 < a.z0 + a.bc;
+}
+
+// DPUTask variants: 3-D inclusive boxes inside the output (nce_cluster_task.cpp:588-608,643-663).
+nce_result_t build_boxes(nce_log_s* log, const nce_cluster_task_desc_t* t, const TensorDev& in, const TensorDev& out, std::vector<Box>* boxes) {
+    if (t->variants == nullptr || t->num_variants == 0) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "task must have at least one DPUTask variant");
+    boxes->clear();
+    for (uint32_t v = 0; v < t->num_variants; ++v) {
+        const nce_dpu_task_t& d = t->variants[v];
+        const int32_t dim[3] = {out.w, out.h, out.c};
+        for (int i = 0; i < 3; ++i)
+            if (d.out_start[i] < 0 || d.out_end[i] < d.out_start[i] || d.out_end[i] >= dim[i])
+                FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "variant %u: out_start/out_end[%d] = %d..%d outside 0..%d", v, i, d.out_start[i], d.out_end[i], dim[i] - 1);
+        if (d.out_start[2] % 16 != 0 || (d.out_end[2] + 1) % 16 != 0)
+            FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "variant %u: channel range %d..%d must cover whole groups of 16", v, d.out_start[2], d.out_end[2]);
+        if (d.mpe_mode < NCE_MPE_VECTOR || d.mpe_mode > NCE_MPE_NOP) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "variant %u: mpe_mode %d", v, d.mpe_mode);
+        if (t->task_type != NCE_TASK_ELTWISE) {
+            // The pad a variant carries is the part of the kernel padding its box touches; the GPU
+            // kernels derive it from global coordinates, so a different value is only reported.
+            const int64_t last_y = (int64_t)d.out_end[1] * t->kernel_strides[0] - t->kernel_pad_top + t->kernel_size[0] - 1;
+            const int64_t last_x = (int64_t)d.out_end[0] * t->kernel_strides[1] - t->kernel_pad_left + t->kernel_size[1] - 1;
+            const int64_t et = std::max<int64_t>(0, t->kernel_pad_top - (int64_t)d.out_start[1] * t->kernel_strides[0]);
+            const int64_t el = std::max<int64_t>(0, t->kernel_pad_left - (int64_t)d.out_start[0] * t->kernel_strides[1]);
+            const int64_t eb = std::max<int64_t>(0, last_y - (in.h - 1));
+            const int64_t er = std::max<int64_t>(0, last_x - (in.w - 1));
+            if (d.pad_top != et || d.pad_bottom != eb || d.pad_left != el || d.pad_right != er)
+                log->add(2, "variant %u: pad {l %d, r %d, t %d, b %d} differs from the geometry {l %lld, r %lld, t %lld, b %lld}; geometry is used",
+                         v, d.pad_left, d.pad_right, d.pad_top, d.pad_bottom, (long long)el, (long long)er, (long long)et, (long long)eb);
+        }
+        Box b;
+        b.x0 = d.out_start[0];
+        b.y0 = d.out_start[1];
+        b.z0 = d.out_start[2];
+        b.bw = d.out_end[0] - d.out_start[0] + 1;
+        b.bh = d.out_end[1] - d.out_start[1] + 1;
+        b.bc = d.out_end[2] - d.out_start[2] + 1;
+        boxes->push_back(b);
+    }
+    // Variants that tile the whole output exactly are one launch over the full box: every output
+    // element is a pure function of its coordinates, so the bytes are the same for any tiling.
+    if (boxes->size() > 1 && boxes->size() <= 1024) {
+        int64_t vol = 0;
+        for (const Box& b : *boxes) vol += box_volume(b);
+        bool exact = vol == (int64_t)out.w * out.h * out.c;
+        for (size_t i = 0; exact && i < boxes->size(); ++i)
+            for (size_t j = i + 1; exact && j < boxes->size(); ++j)
+                if (boxes_overlap((*boxes)[i], (*boxes)[j])) exact = false;
+        if (exact) {
+            Box full = {0, 0, 0, out.w, out.h, out.c};
+            boxes->assign(1, full);
+        }
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t make_plan(nce_log_s* log, const nce_cluster_task_desc_t* t, Plan* plan) {
+    if (t == nullptr) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "task descriptor is null");
+    if (t->flags != 0) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "task flags 0x%x: continued / segmented / compressed / superdense / in-place / permute-quantize / small-kernel tasks are not supported", t->flags);
+    TaskDev& d = plan->dev;
+    memset(&d, 0, sizeof(d));
+    plan->task_type = t->task_type;
+    switch (t->task_type) {
+    case NCE_TASK_CONV:
+    case NCE_TASK_DWCONV:
+    case NCE_TASK_MAXPOOL:
+    case NCE_TASK_AVEPOOL:
+    case NCE_TASK_ELTWISE:
+        break;
+    default:
+        FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "task_type %d is not supported (CONV, DWCONV, MAXPOOL, AVEPOOL, ELTWISE are)", t->task_type);
+    }
+    nce_result_t r;
+    if ((r = check_activation(log, "input", t->input, &d.in)) != NCE_RESULT_SUCCESS) return r;
+    if ((r = check_activation(log, "output", t->output, &d.out)) != NCE_RESULT_SUCCESS) return r;
+
+    const bool has_table = t->weight_table.data != nullptr;
+    if (has_table && (r = check_table(log, t->weight_table, d.out.c, &d)) != NCE_RESULT_SUCCESS) return r;
+
+    if (t->task_type == NCE_TASK_ELTWISE) {
+        // nce_cluster_task.cpp:522-584: no kernel attributes, second input required, same shapes.
+        if (t->kernel_size[0] > 1 || t->kernel_size[1] > 1 || t->kernel_strides[0] > 1 || t->kernel_strides[1] > 1)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ELTWISE must not carry kernel_size / kernel_strides");
+        if (t->kernel_pad_left || t->kernel_pad_right || t->kernel_pad_top || t->kernel_pad_bottom)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ELTWISE must not carry padding");
+        if ((r = check_activation(log, "weights (second eltwise input)", t->weights, &d.in2)) != NCE_RESULT_SUCCESS) return r;
+        if (d.in2.n != d.in.n || d.in2.c != d.in.c || d.in2.h != d.in.h || d.in2.w != d.in.w || d.out.n != d.in.n ||
+            d.out.c != d.in.c || d.out.h != d.in.h || d.out.w != d.in.w)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ELTWISE inputs and output must have the same shape (no broadcast)");
+        if (d.in2.is_signed != d.in.is_signed)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ELTWISE inputs must share the storage type");  // eltwise_utils.cpp:15-65
+        d.ky = d.kx = d.sy = d.sx = 1;
+    } else {
+        if ((r = check_kernel(log, t)) != NCE_RESULT_SUCCESS) return r;
+        if ((r = check_out_shape(log, t, d.in, d.out)) != NCE_RESULT_SUCCESS) return r;
+        d.ky = t->kernel_size[0];
+        d.kx = t->kernel_size[1];
+        d.sy = t->kernel_strides[0];
+        d.sx = t->kernel_strides[1];
+        d.pt = t->kernel_pad_top;
+        d.pl = t->kernel_pad_left;
+    }
+
+    const nce_tensor_t& w = t->weights;
+    if (t->task_type == NCE_TASK_CONV || t->task_type == NCE_TASK_DWCONV) {
+        if (w.data == nullptr) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weights are required");          // nce_cluster_task.cpp:361-378
+        if (!has_table) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weight_table is required");             // nce_cluster_task.cpp:379-398
+        if (!is_8bit(w.dtype)) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "weights: only u8 / i8 storage is supported");
+        int64_t lo, hi;
+        type_range(w.dtype, &lo, &hi);
+        if (w.zero_point < lo || w.zero_point > hi) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weights: zero point %d outside the storage range", w.zero_point);
+        if (((uintptr_t)w.data | (uintptr_t)w.strides_bytes[0]) & 15)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weights: every weight set must start on a 16-byte boundary");  // nce_sparsity.cpp:504-506
+        d.weights = static_cast<const uint8_t*>(w.data);
+        d.w_stride_oc = w.strides_bytes[0];
+        d.w_is_signed = w.dtype == NCE_DT_I8;
+        d.w_zp = w.zero_point;
+    }
+    if (t->task_type == NCE_TASK_CONV) {
+        // OYXI: [OC, IC, KY, KX] logical, IC innermost in memory (nce_cluster_task.cpp:418-433).
+        if (w.dims[0] != d.out.c || w.dims[1] != d.in.c || w.dims[2] != d.ky || w.dims[3] != d.kx)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weights dims [%lld,%lld,%lld,%lld] do not match [OC %d, IC %d, KY %d, KX %d]",
+                 (long long)w.dims[0], (long long)w.dims[1], (long long)w.dims[2], (long long)w.dims[3], d.out.c, d.in.c, d.ky, d.kx);
+        if (w.strides_bytes[1] != 1 || w.strides_bytes[3] != d.in.c || w.strides_bytes[2] != (int64_t)d.kx * d.in.c ||
+            w.strides_bytes[0] < (int64_t)d.ky * d.kx * d.in.c)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "weights must be OYXI with compact weight sets");
+    } else if (t->task_type == NCE_TASK_DWCONV) {
+        // [C, pad16(KY*KX), 1, 1]: one row per channel (const_utils.cpp:216-243; nce_depth_convolution.cpp:93-108).
+        if (d.out.c != d.in.c) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "DWCONV: output channels %d must equal input channels %d", d.out.c, d.in.c);
+        if (w.dims[0] != d.in.c || w.dims[1] < (int64_t)d.ky * d.kx || w.dims[1] % 16 != 0 || w.dims[2] != 1 || w.dims[3] != 1)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "DWCONV weights must be [C, pad16(KY*KX), 1, 1], got [%lld,%lld,%lld,%lld]",
+                 (long long)w.dims[0], (long long)w.dims[1], (long long)w.dims[2], (long long)w.dims[3]);
+        if (w.strides_bytes[1] != 1 || w.strides_bytes[0] < w.dims[1]) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "DWCONV weight rows must be compact");
+    } else if (t->task_type == NCE_TASK_MAXPOOL || t->task_type == NCE_TASK_AVEPOOL) {
+        if (d.out.c != d.in.c) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "pooling: output channels %d must equal input channels %d", d.out.c, d.in.c);
+        if (t->task_type == NCE_TASK_MAXPOOL) {
+            if (t->output.dtype != t->input.dtype) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "MAXPOOL: input and output storage types must match");
+            d.table = nullptr;  // no scale, no bias on this path
+        }
+    }
+
+    if ((r = build_ppe(log, t, t->output, d.table != nullptr, &d.ppe)) != NCE_RESULT_SUCCESS) return r;
+    return build_boxes(log, t, d.in, d.out, &plan->boxes);
+}
+
+nce_result_t launch_plan(nce_executor_s* ex, const Plan& plan, hipStream_t stream) {
+    for (const Box& b : plan.boxes) {
+        hipError_t e = hipSuccess;
+        switch (plan.task_type) {
+        case NCE_TASK_CONV: e = nce::launch_conv(plan.dev, b, stream); break;
+        case NCE_TASK_DWCONV: e = nce::launch_dwconv(plan.dev, b, stream); break;
+        case NCE_TASK_MAXPOOL: e = nce::launch_pool(plan.dev, b, true, stream); break;
+        case NCE_TASK_AVEPOOL: e = nce::launch_pool(plan.dev, b, false, stream); break;
+        case NCE_TASK_ELTWISE: e = nce::launch_eltwise(plan.dev, b, stream); break;
+        }
+        if (e != hipSuccess) {
+            ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
+            return NCE_RESULT_ERROR_UNKNOWN;
+        }
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+}  // namespace
+
+struct nce_task_list_s {
+    nce_executor_s* ex = nullptr;
+    std::vector<Plan> plans;
+};
+
+extern "C" {
+
+nce_result_t nceGetVersion(uint32_t* major, uint32_t* minor) {
+    if (major == nullptr || minor == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    *major = NCE_HIP_VERSION_MAJOR;
+    *minor = NCE_HIP_VERSION_MINOR;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* executor, nce_log_handle_t* log) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    *executor = nullptr;
+    if (log) *log = nullptr;
+    nce_log_s* lg = new (std::nothrow) nce_log_s;
+    nce_executor_s* ex = new (std::nothrow) nce_executor_s;
+    if (lg == nullptr || ex == nullptr) {
+        delete lg;
+        delete ex;
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    }
+    lg->level = desc.log_level;
+    ex->log = lg;
+    ex->device = desc.device_id;
+    if (desc.device_id >= 0) {
+        int count = 0;
+        const hipError_t e = hipGetDeviceCount(&count);
+        if (e != hipSuccess || desc.device_id >= count) {
+            if (desc.log_level >= 1)
+                fprintf(stderr, "nceExecutorCreate: no usable HIP device %d (%d visible): %s\n", desc.device_id, count,
+                        hipGetErrorString(e));
+            delete ex;
+            delete lg;
+            return NCE_RESULT_ERROR_UNSUPPORTED;
+        }
+    }
+    *executor = ex;
+    if (log) *log = lg;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceExecutorDestroy(nce_executor_handle_t executor) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    delete executor->log;
+    delete executor;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceClusterTaskValidate(nce_executor_handle_t executor, const nce_cluster_task_desc_t* task) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    try {
+        Plan plan;
+        return make_plan(executor->log, task, &plan);
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (...) {
+        return NCE_RESULT_ERROR_UNKNOWN;
+    }
+}
+
+nce_result_t nceClusterTaskEnqueue(nce_executor_handle_t executor, const nce_cluster_task_desc_t* task, void* hip_stream) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    try {
+        Plan plan;
+        const nce_result_t r = make_plan(executor->log, task, &plan);
+        if (r != NCE_RESULT_SUCCESS) return r;
+        if (executor->device < 0) {
+            executor->log->add(1, "executor was created without a device (device_id < 0): it can validate, not launch");
+            return NCE_RESULT_ERROR_UNSUPPORTED;
+        }
+        if (hipSetDevice(executor->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
+        return launch_plan(executor, plan, static_cast<hipStream_t>(hip_stream));
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (...) {
+        return NCE_RESULT_ERROR_UNKNOWN;
+    }
+}
+
+nce_result_t nceTaskListCreate(nce_executor_handle_t executor, nce_task_list_handle_t* list) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (list == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    *list = new (std::nothrow) nce_task_list_s;
+    if (*list == nullptr) return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    (*list)->ex = executor;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_task_desc_t* task) {
+    if (list == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    try {
+        Plan plan;
+        const nce_result_t r = make_plan(list->ex->log, task, &plan);
+        if (r != NCE_RESULT_SUCCESS) return r;
+        list->plans.push_back(std::move(plan));
+        return NCE_RESULT_SUCCESS;
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (...) {
+        return NCE_RESULT_ERROR_UNKNOWN;
+    }
+}
+
+nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
+    if (list == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (list->ex->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
+    if (hipSetDevice(list->ex->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
+    for (const Plan& p : list->plans) {
+        const nce_result_t r = launch_plan(list->ex, p, static_cast<hipStream_t>(hip_stream));
+        if (r != NCE_RESULT_SUCCESS) return r;
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceTaskListDestroy(nce_task_list_handle_t list) {
+    if (list == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    delete list;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceExecutorSynchronize(nce_executor_handle_t executor, void* hip_stream) {
+    if (executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (executor->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
+    if (hipSetDevice(executor->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
+    const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) {
+        executor->log->add(1, "synchronize failed: %s", hipGetErrorString(e));
+        return NCE_RESULT_ERROR_UNKNOWN;
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceLogHandleGetString(nce_log_handle_t log, size_t* size, char* buf) {
+    if (log == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (size == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lk(log->mu);
+    if (buf == nullptr) {
+        *size = log->text.size() + 1;
+        return NCE_RESULT_SUCCESS;
+    }
+    if (*size == 0) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    const size_t n = std::min(*size - 1, log->text.size());
+    memcpy(buf, log->text.data(), n);
+    buf[n] = '\0';
+    *size = n + 1;
+    log->text.clear();
+    return NCE_RESULT_SUCCESS;
+}
+
+}  // extern "C"

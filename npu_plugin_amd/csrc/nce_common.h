@@ -1,0 +1,56 @@
+// Internal declarations shared by the host side (nce_api.cpp) and the kernel files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nce_hip.h"
+
+namespace nce {
+
+// Epilogue parameters in the form the kernels consume. The host folds the descriptor's clamp
+// domain, the output zero point and the storage range of the output type into one clamp that is
+// applied BEFORE the zero point is added: y = med3(y, lo, hi) + zp. With L <= H this is identical
+// to "add zp, clamp to [L, H], saturate to the type" because every bound stays far inside int32.
+struct PpeDev {
+    int32_t lo, hi;        // clamp in the zero-point-free domain
+    int32_t zp_out;        // output zero point (0 for MAXPOOL)
+    int32_t prelu_mult;    // multiplier for negative values (1,0 = identity; 0,0 = ReLU)
+    int32_t prelu_shift;
+    int32_t round_mode;    // nce_round_mode_t
+    int32_t quant_mult;    // scale when there is no weight table (ELTWISE / AVEPOOL)
+    int32_t quant_shift;
+    int32_t in1_mult, in2_mult;  // ELTWISE per-input multipliers (1,1 when absent)
+};
+
+// An output sub-box (one DPUTask variant, or the whole tensor) in output coordinates.
+struct Box {
+    int32_t x0, y0, z0;  // inclusive start
+    int32_t bw, bh, bc;  // extent in x (W), y (H), z (C)
+};
+
+struct TensorDev {
+    uint8_t* data;
+    int64_t sn, sh, sw;  // strides in bytes for N, H, W (C is compact)
+    int32_t n, c, h, w;
+    int32_t is_signed;   // storage type i8
+    int32_t zp;
+};
+
+struct TaskDev {
+    TensorDev in, in2, out;  // in2: second eltwise input
+    const uint8_t* weights;
+    int64_t w_stride_oc;     // bytes between weight sets (conv) / per-channel rows (depthwise)
+    int32_t w_is_signed, w_zp;
+    const int32_t* table;    // weight table rows of 4 x int32, or nullptr
+    int64_t table_stride;    // int32 elements between rows
+    int32_t ky, kx, sy, sx, pt, pl;
+    PpeDev ppe;
+};
+
+hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);
+hipError_t launch_pool(const TaskDev& t, const Box& box, bool is_max, hipStream_t stream);
+hipError_t launch_dwconv(const TaskDev& t, const Box& box, hipStream_t stream);
+hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream);
+
+}  // namespace nce

@@ -1,0 +1,325 @@
+// CONV task (ZMajor: NHWC activations, OYXI weights) as an implicit GEMM on the gfx950 matrix
+// cores: D[oc][pixel] += W[oc][k] * A[pixel][k], k = (ky, kx, ic) with ic innermost - the order
+// both tensors already have in memory, so a 16-byte MFMA operand is 16 consecutive input channels
+// of one tap. v_mfma_i32_32x32x32_i8 accumulates in int32; the PPE runs on the accumulators in
+// registers and each lane stores 16 consecutive output channels of one pixel with one 128-bit store.
+//
+// Semantics: src/vpux_compiler/src/dialect/VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc
+//   :834-882  activations: zero point removed before the MAC (mpe_actbias), padding contributes 0
+//   :884-945  weights: zero point removed (mpe_wtbias)
+//   :1952-2045 PPE scale from the weight table (ppe_scale_override = 0 for CONV)
+//
+// The matrix cores multiply signed bytes. u8 operands are re-biased by 128 (x ^ 0x80) and the
+// difference between 128 and the real zero point is restored exactly in the epilogue:
+//   sum (a-zpa)(w-zpw) = sum a'w' + da * sum w' + dw * (sum a' + K*da),  a' = a-offa, da = offa-zpa ...
+// Out-of-image taps are filled with the byte zp_a, so that (a' + da) = 0 there.
+#include "nce_ppe_device.h"
+
+namespace nce {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BN = 64;    // output channels per workgroup
+constexpr int ROW = 80;   // LDS row pitch: 64 bytes of K + 16 bytes of padding against bank conflicts
+constexpr int NTHREADS = 256;
+
+struct ConvArgs {
+    const uint8_t* in;
+    int64_t in_sn, in_sh, in_sw;
+    int32_t H, W;
+    const uint8_t* w;
+    int64_t w_soc;
+    const int32_t* table;
+    int64_t table_stride;
+    uint8_t* out;
+    int64_t out_sn, out_sh, out_sw;
+    int32_t x0, y0, z0, bw, bh, bc;
+    int64_t M;  // pixels in the box over all batches
+    int32_t KY, KX, SY, SX, PT, PL;
+    int32_t KG;   // 16-byte groups along K: KY*KX*IC/16
+    int32_t ICG;  // 16-byte groups per tap: IC/16
+    uint32_t a_xor, w_xor;  // 0x80808080 for u8 storage, 0 for i8
+    uint32_t fill;          // out-of-image activation word, re-biased
+    int32_t da, dw;         // (storage offset - zero point) of activations / weights
+    int32_t ktot;           // KY*KX*IC
+    PpeDev ppe;
+};
+
+__device__ __forceinline__ int32_t bytesum(uint4 v) {
+    int32_t s = 0;
+    s = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.w, 0x01010101, s, false);
+    return s;
+}
+
+// PXF = 32-pixel fragments per wavefront; the workgroup tile is (4 * 32 * PXF) pixels x 64 channels.
+template <int PXF>
+__global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
+    constexpr int BM = 128 * PXF;
+    constexpr int NB = 2 * PXF;  // activation rows each thread stages per step
+
+    __shared__ __attribute__((aligned(16))) uint8_t sA[2][BN * ROW];
+    __shared__ __attribute__((aligned(16))) uint8_t sB[2][BM * ROW];
+    __shared__ int32_t sW2[BN], sBias[BN], sWsum[BN];
+    __shared__ int32_t sAsum[BM];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+
+    const int64_t m0 = (int64_t)blockIdx.x * BM;
+    const int32_t oc0 = a.z0 + blockIdx.y * BN;
+    const int32_t noc = min(BN, a.z0 + a.bc - oc0);
+
+    if (tid < BN) {
+        int32_t w2 = 0, b = 0;
+        if (tid < noc) {
+            const int32_t* row = a.table + (int64_t)(oc0 + tid) * a.table_stride;
+            w2 = row[2];
+            b = row[3];
+        }
+        sW2[tid] = w2;
+        sBias[tid] = b;
+        sWsum[tid] = 0;
+    }
+    for (int i = tid; i < BM; i += NTHREADS) sAsum[i] = 0;
+
+    // ---- staging assignment: thread -> (row, 16-byte group) -------------------------------
+    const int grp = tid & 3;
+    const int srow = tid >> 2;  // 0..63
+    const bool w_valid = srow < noc;
+    const uint8_t* w_ptr = a.w + (int64_t)(oc0 + srow) * a.w_soc;
+
+    const uint8_t* b_base[NB];
+    int32_t b_iy0[NB], b_ix0[NB];
+    bool b_valid[NB];
+    const int64_t box_pix = (int64_t)a.bh * a.bw;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        const int64_t p = m0 + srow + 64 * i;
+        b_valid[i] = p < a.M;
+        const int64_t pp = b_valid[i] ? p : 0;
+        const int64_t n = pp / box_pix;
+        const int32_t rem = (int32_t)(pp - n * box_pix);
+        const int32_t by = rem / a.bw;
+        const int32_t bx = rem - by * a.bw;
+        b_base[i] = a.in + n * a.in_sn;
+        b_iy0[i] = (a.y0 + by) * a.SY - a.PT;
+        b_ix0[i] = (a.x0 + bx) * a.SX - a.PL;
+    }
+
+    // position of this thread's group inside K: g = step*4 + grp -> (ky, kx, icg)
+    int32_t g = grp;
+    int32_t icg = grp, kx = 0, ky = 0;
+    while (icg >= a.ICG) {
+        icg -= a.ICG;
+        if (++kx == a.KX) {
+            kx = 0;
+            ++ky;
+        }
+    }
+
+    uint4 regA;
+    uint4 regB[NB];
+    int32_t wsum = 0;
+    int32_t asum[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) asum[i] = 0;
+    const uint4 fill4 = make_uint4(a.fill, a.fill, a.fill, a.fill);
+
+    auto load_step = [&]() {
+        const bool g_valid = g < a.KG;
+        regA = make_uint4(0, 0, 0, 0);
+        if (g_valid && w_valid) {
+            regA = *reinterpret_cast<const uint4*>(w_ptr + (int64_t)g * 16);
+            regA.x ^= a.w_xor;
+            regA.y ^= a.w_xor;
+            regA.z ^= a.w_xor;
+            regA.w ^= a.w_xor;
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const int32_t iy = b_iy0[i] + ky;
+            const int32_t ix = b_ix0[i] + kx;
+            const bool inb = g_valid && b_valid[i] && (uint32_t)iy < (uint32_t)a.H && (uint32_t)ix < (uint32_t)a.W;
+            uint4 v = fill4;
+            if (inb) {
+                v = *reinterpret_cast<const uint4*>(b_base[i] + (int64_t)iy * a.in_sh + (int64_t)ix * a.in_sw +
+                                                    (icg << 4));
+                v.x ^= a.a_xor;
+                v.y ^= a.a_xor;
+                v.z ^= a.a_xor;
+                v.w ^= a.a_xor;
+            }
+            regB[i] = v;
+        }
+        if (a.da != 0) wsum += bytesum(regA);
+        if (a.dw != 0 && g_valid) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) asum[i] += bytesum(regB[i]);
+        }
+        // advance to the next step's group
+        g += 4;
+        icg += 4;
+        while (icg >= a.ICG) {
+            icg -= a.ICG;
+            if (++kx == a.KX) {
+                kx = 0;
+                ++ky;
+            }
+        }
+    };
+    auto store_step = [&](int buf) {
+        *reinterpret_cast<uint4*>(&sA[buf][srow * ROW + grp * 16]) = regA;
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            *reinterpret_cast<uint4*>(&sB[buf][(srow + 64 * i) * ROW + grp * 16]) = regB[i];
+    };
+
+    // ---- accumulators ------------------------------------------------------------------------
+    v16i acc[2][PXF];
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int x = 0; x < PXF; ++x)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[f][x][v] = 0;
+
+    // MFMA row i of the weight operand carries channel 16*((i>>2)&1) + 4*(i>>3) + (i&3), so that the
+    // 16 accumulator registers of a lane are 16 CONSECUTIVE channels (16*half .. 16*half+15).
+    const int a_row = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+    const int b_row0 = wave * 32 * PXF + l32;
+
+    const int nsteps = (a.KG + 3) >> 2;
+    load_step();
+    store_step(0);
+    __syncthreads();
+    for (int step = 0; step < nsteps; ++step) {
+        const int buf = step & 1;
+        const bool more = step + 1 < nsteps;
+        if (more) load_step();
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const int koff = (kk * 2 + half) * 16;
+            v4i fa[2], fb[PXF];
+#pragma unroll
+            for (int f = 0; f < 2; ++f) fa[f] = *reinterpret_cast<const v4i*>(&sA[buf][(32 * f + a_row) * ROW + koff]);
+#pragma unroll
+            for (int x = 0; x < PXF; ++x) fb[x] = *reinterpret_cast<const v4i*>(&sB[buf][(b_row0 + 32 * x) * ROW + koff]);
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int x = 0; x < PXF; ++x)
+                    acc[f][x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[f], fb[x], acc[f][x], 0, 0, 0);
+        }
+        if (more) store_step(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- zero-point corrections (only when a zero point differs from the storage offset) -------
+    if (a.da != 0 || a.dw != 0) {
+        if (a.da != 0) atomicAdd(&sWsum[srow], wsum);
+        if (a.dw != 0) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) atomicAdd(&sAsum[srow + 64 * i], asum[i]);
+        }
+        __syncthreads();
+    }
+
+    // ---- PPE + store -----------------------------------------------------------------------------
+#pragma unroll
+    for (int x = 0; x < PXF; ++x) {
+        const int prow = b_row0 + 32 * x;
+        const int64_t p = m0 + prow;
+        if (p >= a.M) continue;
+        const int64_t n = p / box_pix;
+        const int32_t rem = (int32_t)(p - n * box_pix);
+        const int32_t by = rem / a.bw;
+        const int32_t bx = rem - by * a.bw;
+        uint8_t* dst = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw;
+        const int32_t a_corr = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {
+            const int ocl = 32 * f + 16 * half;
+            if (ocl >= noc) continue;
+            uint32_t wo[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int c = ocl + v;
+                uint32_t av = (uint32_t)acc[f][x][v] + (uint32_t)a_corr;
+                if (a.da != 0) av += (uint32_t)(a.da * sWsum[c]);
+                const int32_t w2 = sW2[c];
+                const int32_t y = ppe_apply((int32_t)av, sBias[c], table_mult(w2), table_shift(w2), a.ppe);
+                wo[v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+            }
+            *reinterpret_cast<uint4*>(dst + oc0 + ocl) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
+    ConvArgs a;
+    a.in = t.in.data;
+    a.in_sn = t.in.sn;
+    a.in_sh = t.in.sh;
+    a.in_sw = t.in.sw;
+    a.H = t.in.h;
+    a.W = t.in.w;
+    a.w = t.weights;
+    a.w_soc = t.w_stride_oc;
+    a.table = t.table;
+    a.table_stride = t.table_stride;
+    a.out = t.out.data;
+    a.out_sn = t.out.sn;
+    a.out_sh = t.out.sh;
+    a.out_sw = t.out.sw;
+    a.x0 = box.x0;
+    a.y0 = box.y0;
+    a.z0 = box.z0;
+    a.bw = box.bw;
+    a.bh = box.bh;
+    a.bc = box.bc;
+    a.M = (int64_t)t.out.n * box.bh * box.bw;
+    a.KY = t.ky;
+    a.KX = t.kx;
+    a.SY = t.sy;
+    a.SX = t.sx;
+    a.PT = t.pt;
+    a.PL = t.pl;
+    a.ICG = t.in.c / 16;
+    a.KG = t.ky * t.kx * a.ICG;
+    a.ktot = t.ky * t.kx * t.in.c;
+    const int32_t off_a = t.in.is_signed ? 0 : 128;
+    const int32_t off_w = t.w_is_signed ? 0 : 128;
+    a.a_xor = t.in.is_signed ? 0u : 0x80808080u;
+    a.w_xor = t.w_is_signed ? 0u : 0x80808080u;
+    a.da = off_a - t.in.zp;
+    a.dw = off_w - t.w_zp;
+    const uint32_t fb = (uint32_t)((t.in.zp - off_a) & 0xFF);
+    a.fill = fb * 0x01010101u;
+    a.ppe = t.ppe;
+    if (a.M == 0 || box.bc == 0) return hipSuccess;
+
+    const unsigned gy = (unsigned)((box.bc + BN - 1) / BN);
+    // Tile 256 pixels per workgroup only when that still leaves at least two workgroups per CU.
+    const int64_t wg256 = ((a.M + 255) / 256) * gy;
+    if (wg256 >= 512) {
+        const int64_t gx = (a.M + 255) / 256;
+        if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+    } else {
+        const int64_t gx = (a.M + 127) / 128;
+        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace nce

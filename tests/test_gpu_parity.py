@@ -1,0 +1,220 @@
+"""Parity of the HIP executor with the CPU oracle, through the C-ABI, bit-exact (integer path)."""
+import numpy as np
+import pytest
+
+import npu_plugin_amd as nce
+from tests import cases as K
+
+pytestmark = pytest.mark.gpu
+
+
+def check(case, executor):
+    print(f"[case] {case.name} in={case.input.shape} out={case.out_shape}", flush=True)
+    want = K.run_oracle(case)
+    got = K.run_hip(case, executor)
+    bad = np.argwhere(want != got)
+    assert bad.size == 0, (f"{case.name}: {len(bad)} of {want.size} bytes differ; first at {bad[0].tolist()} "
+                           f"oracle={want[tuple(bad[0])]} hip={got[tuple(bad[0])]}")
+
+
+# ---- the five task types at small sizes ------------------------------------------------------
+
+def test_cfg1_conv(executor):
+    check(K.cfg1(), executor)
+
+
+def test_cfg2_conv_lrelu_small_batch(executor):
+    check(K.cfg2(n=1), executor)
+
+
+@pytest.mark.parametrize("ic,oc", [(16, 16), (32, 48), (64, 64), (48, 144), (128, 80), (16, 272)])
+def test_conv_channel_shapes(executor, ic, oc):
+    check(K.conv_case(10 + ic + oc, 2, 9, 11, ic, oc), executor)
+
+
+@pytest.mark.parametrize("k,s,pads", [((1, 1), (1, 1), (0, 0, 0, 0)), ((1, 1), (2, 2), (0, 0, 0, 0)),
+                                      ((3, 3), (2, 2), (1, 1, 1, 1)), ((3, 3), (2, 2), (0, 1, 0, 1)),
+                                      ((7, 7), (2, 2), (3, 3, 3, 3)), ((5, 3), (1, 2), (1, 1, 2, 2)),
+                                      ((11, 11), (4, 4), (5, 5, 5, 5)), ((2, 2), (1, 1), (1, 0, 1, 0)),
+                                      ((1, 1), (1, 1), (1, 1, 1, 1)), ((3, 1), (8, 1), (0, 0, 1, 1))])
+def test_conv_kernel_geometry(executor, k, s, pads):
+    check(K.conv_case(100 + k[0] * 13 + s[0], 2, 23, 19, 32, 32, k=k, s=s, pads=pads), executor)
+
+
+@pytest.mark.parametrize("in_signed,w_signed,in_zp,w_zp,out_signed,out_zp", [
+    (False, True, 128, 0, False, 128),   # the benchmark types
+    (False, True, 0, 0, False, 0),
+    (False, True, 3, 0, False, 17),      # zero point away from the storage offset: weight-sum correction
+    (True, True, 0, 0, True, 0),
+    (True, True, -7, 0, True, -128),
+    (False, False, 128, 128, False, 128),
+    (False, False, 121, 127, False, 255),  # both corrections
+    (True, False, 5, 3, False, 9),
+])
+def test_conv_types_and_zero_points(executor, in_signed, w_signed, in_zp, w_zp, out_signed, out_zp):
+    check(K.conv_case(7, 1, 10, 10, 32, 32, in_signed=in_signed, w_signed=w_signed, in_zp=in_zp, w_zp=w_zp,
+                      out_signed=out_signed, out_zp=out_zp), executor)
+
+
+PPE_VARIANTS = [
+    dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255),
+    dict(mode=nce.PPE_NOOP, clamp_low=128, clamp_high=255),                              # ReLU the 37XX way
+    dict(mode=nce.PPE_LRELU, clamp_low=0, clamp_high=255),
+    dict(mode=nce.PPE_LRELUX, clamp_low=0, clamp_high=200),
+    dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14),
+    dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=-5, lrelu_shift=2),
+    dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=2047, lrelu_shift=31),
+    dict(mode=nce.PPE_NOOP, clamp_low=-128, clamp_high=127, clamp_domain=nce.CLAMP_PRE_ZP),
+    dict(mode=nce.PPE_LRELU, clamp_low=0, clamp_high=100, clamp_domain=nce.CLAMP_PRE_ZP),
+    dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255, round_mode=nce.ROUND_HALF_EVEN),
+    dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=3, lrelu_shift=1, round_mode=nce.ROUND_HALF_EVEN),
+    dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255, round_mode=nce.ROUND_NONE),
+    {},                                                                                 # no PPE task at all
+]
+
+
+@pytest.mark.parametrize("ppe", PPE_VARIANTS)
+def test_conv_ppe_variants(executor, ppe):
+    check(K.conv_case(21, 1, 12, 12, 32, 32, ppe=ppe), executor)
+
+
+@pytest.mark.parametrize("scale_lo,scale_hi", [(1e-6, 1e-5), (1e-2, 1e-1), (0.3, 0.9), (1.0, 7.9), (20.0, 255.0)])
+def test_conv_scale_ranges(executor, scale_lo, scale_hi):
+    # small scales -> shift up to 34; large scales -> shift down to 7 and saturating outputs
+    check(K.conv_case(33, 1, 8, 8, 32, 32, scale_lo=scale_lo, scale_hi=scale_hi), executor)
+
+
+def test_dwconv_cfg3_small(executor):
+    check(K.cfg3_dw(n=1), executor)
+
+
+@pytest.mark.parametrize("c,k,s,pads", [(16, (3, 3), (1, 1), (1, 1, 1, 1)), (96, (3, 3), (2, 2), (1, 1, 1, 1)),
+                                        (272, (5, 5), (1, 1), (2, 2, 2, 2)), (32, (11, 11), (3, 3), (5, 5, 5, 5)),
+                                        (48, (2, 3), (2, 1), (1, 1, 0, 1)), (512, (3, 3), (2, 2), (0, 0, 0, 0))])
+def test_dwconv_shapes(executor, c, k, s, pads):
+    check(K.dw_case(5 + c, 2, 21, 17, c, k=k, s=s, pads=pads), executor)
+
+
+@pytest.mark.parametrize("in_signed,w_signed,in_zp,w_zp", [(False, False, 100, 131), (True, True, -3, 0), (True, False, 1, 2)])
+def test_dwconv_types(executor, in_signed, w_signed, in_zp, w_zp):
+    check(K.dw_case(9, 1, 12, 12, 32, in_signed=in_signed, w_signed=w_signed, in_zp=in_zp, w_zp=w_zp,
+                    out_signed=in_signed, out_zp=-5 if in_signed else 77), executor)
+
+
+@pytest.mark.parametrize("is_max", [True, False])
+@pytest.mark.parametrize("k,s,pads", [((3, 3), (2, 2), (1, 1, 1, 1)), ((2, 2), (2, 2), (0, 0, 0, 0)),
+                                      ((3, 3), (1, 1), (1, 1, 1, 1)), ((7, 7), (7, 7), (0, 0, 0, 0))])
+def test_pools(executor, is_max, k, s, pads):
+    check(K.pool_case(3, is_max, 2, 28, 28, 96, k=k, s=s, pads=pads), executor)
+    check(K.pool_case(4, is_max, 1, 14, 14, 32, k=k, s=s, pads=pads, in_signed=True, in_zp=-11, out_zp=4), executor)
+
+
+def test_avgpool_with_weight_table(executor):
+    check(K.pool_case(6, False, 2, 14, 14, 64, with_table=True), executor)
+
+
+def test_maxpool_clamped(executor):
+    check(K.pool_case(8, True, 1, 14, 14, 32, ppe=dict(mode=nce.PPE_NOOP, clamp_low=30, clamp_high=200)), executor)
+
+
+def test_eltwise_cfg4_small(executor):
+    check(K.cfg4(n=2), executor)
+
+
+@pytest.mark.parametrize("kw", [dict(with_in_mult=False, mult=16384, shift=15),
+                                dict(signed=True, zp_a=-3, zp_b=12, out_zp=-100),
+                                dict(with_table=True),
+                                dict(ppe_extra=dict(round_mode=nce.ROUND_HALF_EVEN)),
+                                dict(ppe_extra=dict(mode=nce.PPE_LRELU, clamp_low=128)),
+                                dict(in1_mult=65535, in2_mult=65535, mult=65535, shift=40),
+                                dict(mult=3, shift=0, in1_mult=1, in2_mult=1)])
+def test_eltwise_variants(executor, kw):
+    check(K.eltwise_case(11, 1, 7, 9, 48, **kw), executor)
+
+
+# ---- variants: any tiling of the output box gives the same bytes ---------------------------------
+
+def _tilings(oh, ow, oc):
+    yield [((0, 0, 0), (ow - 1, oh // 2 - 1, oc - 1)), ((0, oh // 2, 0), (ow - 1, oh - 1, oc - 1))]       # split over height
+    yield [((0, 0, 0), (ow - 1, oh - 1, 15)), ((0, 0, 16), (ow - 1, oh - 1, oc - 1))]                     # split over channels
+    yield [((0, 0, 0), (ow // 3, oh - 1, oc - 1)), ((ow // 3 + 1, 0, 0), (ow - 1, oh - 1, oc - 1))]       # split over width
+    yield [((1, 2, 16), (ow - 2, oh - 2, oc - 1))]                                                       # partial cover
+
+
+@pytest.mark.parametrize("which", range(4))
+def test_variant_tilings(executor, which):
+    for maker in (lambda v: K.conv_case(41, 2, 12, 10, 32, 48, variants=v),
+                  lambda v: K.dw_case(42, 2, 24, 20, 48, variants=v),
+                  lambda v: K.pool_case(43, True, 2, 24, 20, 48, variants=v),
+                  lambda v: K.pool_case(44, False, 2, 24, 20, 48, variants=v),
+                  lambda v: K.eltwise_case(45, 2, 12, 10, 48, variants=v)):
+        probe = maker(None)
+        _, oh, ow, oc = probe.out_shape
+        tiling = list(_tilings(oh, ow, oc))[which]
+        case = maker(tiling)
+        # bytes outside the variants must stay untouched: compare against the oracle run on the same
+        # poisoned canvas
+        want = np.full(case.out_shape, 0x5A, dtype=np.uint8)
+        from oracle import nce_oracle
+        nce_oracle.run(K.build_task(case, case.input, case.weights, case.table, want))
+        got = K.run_hip(case, executor)
+        assert np.array_equal(want, got), f"{case.name} tiling {which}"
+        if which < 3:
+            assert np.array_equal(got, K.run_oracle(probe)), "a full tiling must equal the single-variant result"
+
+
+def test_strided_views(executor):
+    """parent_input / parent_output style sub-views: W and H strides larger than the compact ones."""
+    import torch
+    case = K.conv_case(51, 1, 8, 8, 32, 32)
+    want = K.run_oracle(case)
+    big_in = torch.zeros((1, 10, 12, 64), dtype=torch.uint8, device="cuda")
+    big_out = torch.zeros((1, 9, 11, 48), dtype=torch.uint8, device="cuda")
+    view_in = big_in[:, 1:9, 2:10, 16:48]
+    view_in.copy_(torch.from_numpy(case.input).cuda())
+    view_out = big_out[:, 0:8, 1:9, 16:48]
+    w = torch.from_numpy(case.weights).cuda()
+    t = torch.from_numpy(case.table).cuda()
+    task = K.build_task(case, view_in, w, t, view_out)
+    stream = torch.cuda.current_stream().cuda_stream
+    executor.enqueue(task, stream)
+    executor.synchronize(stream)
+    assert np.array_equal(view_out.cpu().numpy(), want)
+    mask = torch.ones_like(big_out, dtype=torch.bool)
+    mask[:, 0:8, 1:9, 16:48] = False
+    assert not big_out[mask].any(), "bytes outside the output view were written"
+
+
+def test_determinism(executor):
+    case = K.cfg2(n=1)
+    first = K.run_hip(case, executor)
+    for _ in range(3):
+        assert np.array_equal(first, K.run_hip(case, executor))
+
+
+def test_task_list_chain(executor):
+    """conv -> maxpool -> eltwise(add with itself) chained through a task list on one stream."""
+    import torch
+    c1 = K.conv_case(61, 2, 16, 16, 32, 32)
+    y1 = K.run_oracle(c1)
+    c2 = K.pool_case(62, True, 2, 16, 16, 32)
+    c2.input = y1
+    y2 = K.run_oracle(c2)
+    c3 = K.eltwise_case(63, 2, 8, 8, 32)
+    c3.input = y2
+    c3.weights = y2
+    y3 = K.run_oracle(c3)
+
+    d1 = K.DeviceCase(c1)
+    d2 = K.DeviceCase(c2)
+    d3 = K.DeviceCase(c3)
+    t2 = K.build_task(c2, d1.output, None, None, d2.output)
+    t3 = K.build_task(c3, d2.output, d2.output, None, d3.output)
+    tl = executor.task_list()
+    for t in (d1.task, t2, t3):
+        tl.append(t)
+    stream = torch.cuda.current_stream().cuda_stream
+    tl.enqueue(stream)
+    executor.synchronize(stream)
+    tl.destroy()
+    assert np.array_equal(d3.output.cpu().numpy(), y3)
