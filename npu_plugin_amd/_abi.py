@@ -153,6 +153,13 @@ def load_library():
         raise RuntimeError(
             f"{LIB_PATH} is missing: build the HIP library first (python -c 'import __graft_entry__ as g; g.build()'). "
             "There is no CPU fallback.")
+    # PyTorch ships its own HIP runtime (same SONAME as the system one). Two HIP runtimes in one process
+    # do not share the GPU, so let torch load its copy first: the dynamic loader then binds this library
+    # to the runtime that also owns the caller's tensors and streams.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
