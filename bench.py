@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the NCE op path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-others] [--no-cpu]
+
+A step is one pass of one task over its batch of synthetic input, already resident in HBM. The K
+timed steps are launched back to back from one task list (one C call), bracketed by
+torch.cuda.synchronize(); HIP events on the launch stream give the average kernel duration used for
+the roofline figure. Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0  # MI355X dense INT8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0    # MI355X HBM3E, GB/s
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); filled
+# per workload once measured, None otherwise.
+MEASURED_TRAFFIC = {}
+
+
+def make_workloads():
+    from npu_plugin_amd import workloads as W
+    return {
+        "cfg2": (W.cfg2, "mfma"),
+        "cfg3_dw": (W.cfg3_dw, "hbm"),
+        "cfg3_maxpool": (W.cfg3_maxpool, "hbm"),
+        "cfg3_avgpool": (W.cfg3_avgpool, "hbm"),
+        "cfg4": (W.cfg4, "hbm"),
+    }
+
+
+def time_task(ex, dc, steps, warmup):
+    """Returns (wall seconds per step, event seconds per step)."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    warm = ex.task_list()
+    for _ in range(max(warmup, 1)):
+        warm.append(dc.task)
+    timed = ex.task_list()
+    for _ in range(steps):
+        timed.append(dc.task)
+    warm.enqueue(stream)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    timed.enqueue(stream)
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    warm.destroy()
+    timed.destroy()
+    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def measure(ex, name, maker, bound, steps, warmup):
+    from npu_plugin_amd import workloads as W
+    case = maker()
+    dc = W.DeviceCase(case)
+    wall, ev = time_task(ex, dc, steps, warmup)
+    ops, nbytes = case.ops(), case.algorithmic_bytes()
+    if bound == "mfma":
+        value, unit = ops / wall / 1e9, "GOPS"
+        roof = {"bound": "mfma", "achieved": ops / ev / 1e12, "peak": PEAK_INT8_TOPS / 1.0, "unit": "TOP/s"}
+        roof["peak"] = PEAK_INT8_TOPS
+        roof["achieved"] = ops / ev / 1e12
+    else:
+        value, unit = nbytes / wall / 1e9, "GB/s"
+        roof = {"bound": "hbm", "achieved": nbytes / ev / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC.get(name)
+    roof["kernel_us"] = ev * 1e6
+    return case, {"workload": case.name, "value": value, "unit": unit, "ms_per_step": wall * 1e3, "ops_per_step": ops,
+                  "bytes_per_step": nbytes, "roofline": roof}
+
+
+def cpu_baseline(case, bound, budget_s=12.0):
+    """The CPU oracle (a port of the reference's semantics; the reference itself has no executable
+    arithmetic for this path) timed on the host cores, on whole passes of the same workload."""
+    from oracle import nce_oracle
+    from tests.cases import run_oracle
+    cores = min(16, nce_oracle.lib().nce_oracle_max_threads())
+    run_oracle(case, cores)  # warm
+    n, t0 = 0, time.perf_counter()
+    while True:
+        run_oracle(case, cores)
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or n >= 50:
+            break
+    per = dt / n
+    if bound == "mfma":
+        v, unit = case.ops() / per / 1e9, "GOPS"
+    else:
+        v, unit = case.algorithmic_bytes() / per / 1e9, "GB/s"
+    return {"value": v, "unit": unit, "cores": cores, "kind": "port",
+            "sample": f"{n} full passes of {case.name} ({per * 1e3:.1f} ms each)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported (no collectives, no sharding).")
+
+    import torch  # noqa: F401  (device memory and streams)
+
+    import npu_plugin_amd as nce
+    workloads = make_workloads()
+    if args.workload not in workloads:
+        sys.exit(f"unknown workload {args.workload}; choose from {sorted(workloads)}")
+    ex = nce.Executor(device_id=0, log_level=1)
+
+    maker, bound = workloads[args.workload]
+    case, main_res = measure(ex, args.workload, maker, bound, args.steps, args.warmup)
+    line = {
+        "metric": "INT8 GOPS & % MFMA peak (conv); GB/s & % HBM peak (dw/pool/eltwise)",
+        "value": main_res["value"],
+        "unit": main_res["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 (u8 x i8 -> i32 accumulate, integer PPE)",
+        "data": "synthetic (seeded uniform u8 activations, i8 weights, random per-channel mult/shift tables)",
+        "config": {"workload": case.name, "ops_per_step": main_res["ops_per_step"], "bytes_per_step": main_res["bytes_per_step"]},
+        "roofline": main_res["roofline"],
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(case, bound)
+    if not args.no_others:
+        others = {}
+        for name, (mk, bd) in workloads.items():
+            if name == args.workload:
+                continue
+            _, r = measure(ex, name, mk, bd, args.steps, args.warmup)
+            others[name] = r
+        line["other_workloads"] = others
+    ex.destroy()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
