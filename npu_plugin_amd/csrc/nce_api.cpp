@@ -193,6 +193,14 @@ nce_result_t build_ppe(nce_log_s* log, const nce_cluster_task_desc_t* t, const n
     d->lo = (int32_t)(clamp64(lo, tlo, thi) - zp);
     d->hi = (int32_t)(clamp64(hi, tlo, thi) - zp);
     d->zp_out = (int32_t)zp;
+    if (!is_max && d->prelu_mult == 0) {
+        // slope 0 (ReLU): negative values become 0 before the clamp, which is the clamp with its
+        // lower bound raised to 0 - the kernels then skip the PReLU step altogether
+        d->prelu_mult = 1;
+        d->prelu_shift = 0;
+        if (d->lo < 0) d->lo = 0;
+        if (d->hi < d->lo) d->lo = d->hi;
+    }
 
     d->quant_mult = 1;
     d->quant_shift = 0;

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
 
     __shared__ __attribute__((aligned(16))) uint8_t sA[2][BN * ROW];
     __shared__ __attribute__((aligned(16))) uint8_t sB[2][BM * ROW];
-    __shared__ int32_t sW2[BN], sBias[BN], sWsum[BN];
+    __shared__ int32_t sW2[BN], sBias[BN], sWsum[BN], sCorr[BN];
+    __shared__ double sM[BN], sBc[BN];
     __shared__ int32_t sAsum[BM];
 
     const int tid = threadIdx.x;
@@ -222,7 +223,9 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         __syncthreads();
     }
 
-    // ---- zero-point corrections (only when a zero point differs from the storage offset) -------
+    // ---- per-channel epilogue constants ------------------------------------------------------
+    // Zero-point corrections (only when a zero point differs from the storage offset): the
+    // weight-sum term is constant per channel and goes into B; the activation-sum term is per pixel.
     if (a.da != 0 || a.dw != 0) {
         if (a.da != 0) atomicAdd(&sWsum[srow], wsum);
         if (a.dw != 0) {
@@ -231,35 +234,73 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         }
         __syncthreads();
     }
+    int bad_shift = 0, small_shift = 0;
+    if (tid < BN) {
+        const int32_t w2 = sW2[tid];
+        const int32_t mult = table_mult(w2), shift = table_shift(w2);
+        const int32_t corr = a.da * sWsum[tid];  // |da| <= 255, |sum w'| < 2^23
+        const double M = ppe_scale_M(mult, shift);
+        sM[tid] = M;
+        sBc[tid] = __builtin_fma((double)corr, M, ppe_scale_B(sBias[tid], M, shift, a.ppe.round_mode));
+        sCorr[tid] = corr;
+        bad_shift = shift > kMaxF64Shift;
+        small_shift = shift < kNoSatShift;
+    }
+    const bool use_int = __syncthreads_or(bad_shift) != 0;
+    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    const PpeF64 pu = ppe_f64_setup(a.ppe, may_sat);
 
     // ---- PPE + store -----------------------------------------------------------------------------
+    uint8_t* dst[PXF];
+    int32_t a_corr[PXF];
+    bool p_valid[PXF];
 #pragma unroll
     for (int x = 0; x < PXF; ++x) {
         const int prow = b_row0 + 32 * x;
         const int64_t p = m0 + prow;
-        if (p >= a.M) continue;
-        const int64_t n = p / box_pix;
-        const int32_t rem = (int32_t)(p - n * box_pix);
+        p_valid[x] = p < a.M;
+        const int64_t pp = p_valid[x] ? p : 0;
+        const int64_t n = pp / box_pix;
+        const int32_t rem = (int32_t)(pp - n * box_pix);
         const int32_t by = rem / a.bw;
         const int32_t bx = rem - by * a.bw;
-        uint8_t* dst = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw;
-        const int32_t a_corr = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
+        dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+        a_corr[x] = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
+    }
 #pragma unroll
-        for (int f = 0; f < 2; ++f) {
-            const int ocl = 32 * f + 16 * half;
-            if (ocl >= noc) continue;
-            uint32_t wo[4] = {0, 0, 0, 0};
+    for (int f = 0; f < 2; ++f) {
+        const int ocl = 32 * f + 16 * half;
+        if (ocl >= noc) continue;
+        uint32_t wo[PXF][4];
+#pragma unroll
+        for (int x = 0; x < PXF; ++x) wo[x][0] = wo[x][1] = wo[x][2] = wo[x][3] = 0;
+        if (!use_int) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const double M = sM[ocl + v], B = sBc[ocl + v];
+#pragma unroll
+                for (int x = 0; x < PXF; ++x) {
+                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)a_corr[x]);
+                    const int32_t y = ppe_apply_f64(av, M, B, pu);
+                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+                }
+            }
+        } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int c = ocl + v;
-                uint32_t av = (uint32_t)acc[f][x][v] + (uint32_t)a_corr;
-                if (a.da != 0) av += (uint32_t)(a.da * sWsum[c]);
                 const int32_t w2 = sW2[c];
-                const int32_t y = ppe_apply((int32_t)av, sBias[c], table_mult(w2), table_shift(w2), a.ppe);
-                wo[v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+#pragma unroll
+                for (int x = 0; x < PXF; ++x) {
+                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)a_corr[x] + (uint32_t)sCorr[c]);
+                    const int32_t y = ppe_apply(av, sBias[c], table_mult(w2), table_shift(w2), a.ppe);
+                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+                }
             }
-            *reinterpret_cast<uint4*>(dst + oc0 + ocl) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
         }
+#pragma unroll
+        for (int x = 0; x < PXF; ++x)
+            if (p_valid[x]) *reinterpret_cast<uint4*>(dst[x] + ocl) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
     }
 }
 

@@ -3,7 +3,9 @@
 // (per-input multipliers elop_scale_a/b) and :1651-1757 (scale override from the PPE task).
 //
 // Memory-bound: each lane moves one 16-byte channel group of both inputs and of the output
-// (global_load_dwordx4 x2, global_store_dwordx4 x1), 48 algorithmic bytes per 16 outputs.
+// (global_load_dwordx4 x2, global_store_dwordx4 x1), 48 algorithmic bytes per 16 outputs. The
+// requantize runs in FP64 (exact, see nce_ppe_device.h); per-channel tables and shifts above 52
+// take the integer path.
 #include "nce_ppe_device.h"
 
 namespace nce {
@@ -14,16 +16,29 @@ __device__ __forceinline__ int32_t byte_at(uint32_t w, int i) {
     return SIGNED ? (int32_t)(int8_t)(w >> (8 * i)) : (int32_t)((w >> (8 * i)) & 0xFFu);
 }
 
-template <bool FLAT, bool HAS_TABLE, bool A_SIGNED, bool B_SIGNED>
-__global__ __launch_bounds__(256) void eltwise_kernel(TaskDev t, Box box, int64_t nchunks) {
+struct EltArgs {
+    TaskDev t;
+    Box box;
+    int64_t nchunks;
+    double M, B;  // uniform scale constants (no weight table)
+    int32_t c0;   // -(in1_mult * zp_a + in2_mult * zp_b)
+    int32_t may_sat;
+};
+
+// PATH 0: FP64 with uniform scale. PATH 1: integer, uniform scale. PATH 2: integer, per-channel table.
+template <bool FLAT, int PATH, bool SIGNED>
+__global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
+    const TaskDev& t = a.t;
+    const Box& box = a.box;
     const int32_t cgroups = box.bc >> 4;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < nchunks;
+    const PpeF64 pu = ppe_f64_setup(t.ppe, a.may_sat != 0);
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < a.nchunks;
          idx += (int64_t)gridDim.x * blockDim.x) {
         int64_t off_a, off_b, off_o;
-        int32_t oc;
+        int32_t oc = 0;
         if (FLAT) {
             off_a = off_b = off_o = idx << 4;
-            oc = (int32_t)(idx % cgroups) << 4;
+            if (PATH == 2) oc = (int32_t)(idx % cgroups) << 4;
         } else {
             int64_t r = idx;
             const int32_t cg = (int32_t)(r % cgroups);
@@ -43,24 +58,22 @@ __global__ __launch_bounds__(256) void eltwise_kernel(TaskDev t, Box box, int64_
         const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
         const uint32_t wb[4] = {vb.x, vb.y, vb.z, vb.w};
         uint32_t wo[4];
-        // c0 folds both zero points: m1*(a-zpa) + m2*(b-zpb) = m1*a + m2*b + c0. |c0| < 2^26.
-        const int32_t c0 = -(t.ppe.in1_mult * t.in.zp + t.ppe.in2_mult * t.in2.zp);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             uint32_t packed = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int32_t a = byte_at<A_SIGNED>(wa[d], i);
-                const int32_t b = byte_at<B_SIGNED>(wb[d], i);
-                const int32_t acc = t.ppe.in1_mult * a + t.ppe.in2_mult * b + c0;
-                int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
-                if (HAS_TABLE) {
+                // |acc| < 2^26: 16-bit multipliers times 9-bit values, twice, plus c0
+                const int32_t acc = t.ppe.in1_mult * byte_at<SIGNED>(wa[d], i) + t.ppe.in2_mult * byte_at<SIGNED>(wb[d], i) + a.c0;
+                int32_t y;
+                if (PATH == 0) {
+                    y = ppe_apply_f64(acc, a.M, a.B, pu);
+                } else if (PATH == 1) {
+                    y = ppe_apply(acc, 0, t.ppe.quant_mult, t.ppe.quant_shift, t.ppe);
+                } else {
                     const int32_t* row = t.table + (int64_t)(oc + 4 * d + i) * t.table_stride;
-                    mult = table_mult(row[2]);
-                    shift = table_shift(row[2]);
-                    bias = row[3];
+                    y = ppe_apply(acc, row[3], table_mult(row[2]), table_shift(row[2]), t.ppe);
                 }
-                const int32_t y = ppe_apply(acc, bias, mult, shift, t.ppe);
                 packed |= ((uint32_t)y & 0xFFu) << (8 * i);
             }
             wo[d] = packed;
@@ -73,36 +86,40 @@ bool is_dense_nhwc(const TensorDev& x) {
     return x.sw == x.c && x.sh == (int64_t)x.w * x.c && x.sn == (int64_t)x.h * x.w * x.c;
 }
 
-template <bool FLAT, bool HAS_TABLE>
-void launch_signed(const TaskDev& t, const Box& box, int64_t nchunks, int grid, hipStream_t s) {
-    const int sel = (t.in.is_signed ? 2 : 0) | (t.in2.is_signed ? 1 : 0);
-    switch (sel) {
-    case 0: hipLaunchKernelGGL((eltwise_kernel<FLAT, HAS_TABLE, false, false>), dim3(grid), dim3(256), 0, s, t, box, nchunks); break;
-    case 1: hipLaunchKernelGGL((eltwise_kernel<FLAT, HAS_TABLE, false, true>), dim3(grid), dim3(256), 0, s, t, box, nchunks); break;
-    case 2: hipLaunchKernelGGL((eltwise_kernel<FLAT, HAS_TABLE, true, false>), dim3(grid), dim3(256), 0, s, t, box, nchunks); break;
-    default: hipLaunchKernelGGL((eltwise_kernel<FLAT, HAS_TABLE, true, true>), dim3(grid), dim3(256), 0, s, t, box, nchunks); break;
-    }
+template <bool FLAT, int PATH>
+void launch_signed(const EltArgs& a, int grid, hipStream_t s) {
+    if (a.t.in.is_signed) hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH, true>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH, false>), dim3(grid), dim3(256), 0, s, a);
+}
+
+template <bool FLAT>
+void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
+    if (path == 0) launch_signed<FLAT, 0>(a, grid, s);
+    else if (path == 1) launch_signed<FLAT, 1>(a, grid, s);
+    else launch_signed<FLAT, 2>(a, grid, s);
 }
 
 }  // namespace
 
 hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) {
-    const int64_t nchunks = (int64_t)t.out.n * box.bh * box.bw * (box.bc >> 4);
-    if (nchunks == 0) return hipSuccess;
+    EltArgs a;
+    a.t = t;
+    a.box = box;
+    a.nchunks = (int64_t)t.out.n * box.bh * box.bw * (box.bc >> 4);
+    if (a.nchunks == 0) return hipSuccess;
     const bool full = box.x0 == 0 && box.y0 == 0 && box.z0 == 0 && box.bw == t.out.w && box.bh == t.out.h &&
                       box.bc == t.out.c;
     const bool flat = full && is_dense_nhwc(t.in) && is_dense_nhwc(t.in2) && is_dense_nhwc(t.out);
-    const bool has_table = t.table != nullptr;
-    int64_t blocks = (nchunks + 255) / 256;
+    a.c0 = -(t.ppe.in1_mult * t.in.zp + t.ppe.in2_mult * t.in2.zp);
+    const int shift = t.ppe.quant_shift;
+    a.M = ldexp((double)t.ppe.quant_mult, -shift);
+    a.B = (t.ppe.round_mode == NCE_ROUND_HALF_UP && shift > 0) ? 0.5 : 0.0;
+    a.may_sat = shift < 18;
+    const int path = t.table != nullptr ? 2 : (shift > 52 ? 1 : 0);
+    int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    const int grid = (int)blocks;
-    if (flat) {
-        if (has_table) launch_signed<true, true>(t, box, nchunks, grid, stream);
-        else launch_signed<true, false>(t, box, nchunks, grid, stream);
-    } else {
-        if (has_table) launch_signed<false, true>(t, box, nchunks, grid, stream);
-        else launch_signed<false, false>(t, box, nchunks, grid, stream);
-    }
+    if (flat) launch_path<true>(a, path, (int)blocks, stream);
+    else launch_path<false>(a, path, (int)blocks, stream);
     return hipGetLastError();
 }
 

@@ -2,13 +2,25 @@
 // Order of operations follows the reference's register programming
 // (src/vpux_compiler/src/dialect/VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc:511-542
 // for PReLU / zero point, :1952-2045 for scale, clamp and rounding registers):
-//   x = acc + bias ; x = round_shift(x * mult, shift) ; negative x: x = round_shift(x * prelu_mult,
-//   prelu_shift) ; clamp ; + output zero point ; store as u8 / i8.
+//   x = acc + bias ; x = round_shift(x * mult, shift) ; saturate to int32 ;
+//   negative x: x = round_shift(x * prelu_mult, prelu_shift) ; saturate ; clamp ; + zero point.
+//
+// Two implementations of the same function:
+//   * ppe_apply      - 64-bit integer arithmetic, any shift 0..63.
+//   * ppe_apply_f64  - the same value through FP64, which gfx950 issues at full rate while 64-bit
+//                      integer multiplies and shifts do not. Exact, not approximate: with
+//                      M = mult * 2^-shift and B = bias * M + 1/2, the quantity acc * M + B equals
+//                      N / 2^shift for an integer |N| < 2^53 whenever shift <= 52, so one FMA
+//                      returns it without rounding and floor() (or rint() for ties-to-even) is the
+//                      integer pipeline's rounding shift. Shifts above 52 take the integer path.
 #pragma once
 
 #include "nce_common.h"
 
 namespace nce {
+
+constexpr int kMaxF64Shift = 52;  // largest shift for which the FP64 formulation is exact
+constexpr int kNoSatShift = 18;   // |x * mult| < 2^48, so >> 18 or more cannot leave int32
 
 __device__ __forceinline__ int64_t rshift_round(int64_t p, int32_t s, int32_t mode) {
     if (s <= 0) return p;
@@ -33,8 +45,7 @@ __device__ __forceinline__ int32_t table_shift(int32_t w2) {
     return (int32_t)(((uint32_t)w2 >> 8) & 0x3Fu);
 }
 
-// Full-generality epilogue for one accumulator. Returns the value to store (already in the output
-// type's range), as int32.
+// Integer path. Returns the value to store (already in the output type's range).
 __device__ __forceinline__ int32_t ppe_apply(int32_t acc, int32_t bias, int32_t mult, int32_t shift,
                                              const PpeDev& p) {
     int64_t x = (int64_t)acc + (int64_t)bias;
@@ -45,16 +56,62 @@ __device__ __forceinline__ int32_t ppe_apply(int32_t acc, int32_t bias, int32_t 
     return y + p.zp_out;
 }
 
-// Same result as ppe_apply when 1 <= shift, rounding is HALF_UP and |result| cannot leave int32
-// (shift >= 17 guarantees it: |x * mult| < 2^48). c = bias * mult + 2^(shift-1) is precomputed per
-// output channel so the requantize step is one 64-bit multiply-add and one 64-bit shift.
-__device__ __forceinline__ int32_t ppe_apply_fast(int32_t acc, int32_t mult, int32_t shift, int64_t c,
-                                                  const PpeDev& p) {
-    int32_t y = (int32_t)(((int64_t)acc * (int64_t)mult + c) >> shift);
-    if (y < 0 && !(p.prelu_mult == 1 && p.prelu_shift == 0))
-        y = sat_i32(rshift_round((int64_t)y * (int64_t)p.prelu_mult, p.prelu_shift, NCE_ROUND_HALF_UP));
-    y = y < p.lo ? p.lo : (y > p.hi ? p.hi : y);
-    return y + p.zp_out;
+// ---- FP64 path ------------------------------------------------------------------------------
+
+// Per-channel constants: M = mult * 2^-shift, B = bias * M + (1/2 when rounding half-up and shift > 0).
+__device__ __forceinline__ double ppe_scale_M(int32_t mult, int32_t shift) {
+    return __builtin_ldexp((double)mult, -shift);
+}
+__device__ __forceinline__ double ppe_scale_B(int32_t bias, double M, int32_t shift, int32_t round_mode) {
+    return __builtin_fma((double)bias, M, (round_mode == NCE_ROUND_HALF_UP && shift > 0) ? 0.5 : 0.0);
+}
+
+// Wavefront-uniform part of the FP64 epilogue.
+struct PpeF64 {
+    double pm, pc;   // PReLU slope as prelu_mult * 2^-prelu_shift and its rounding constant
+    int32_t lo, hi, zp;
+    bool even;       // ties-to-even (rint) instead of floor
+    bool sat;        // requantized value may leave int32: clamp it (some shift < kNoSatShift)
+    bool prelu;      // slope differs from identity
+    bool prelu_sat;  // slope result may leave int32
+};
+
+__device__ __forceinline__ PpeF64 ppe_f64_setup(const PpeDev& p, bool may_saturate) {
+    PpeF64 u;
+    u.pm = __builtin_ldexp((double)p.prelu_mult, -p.prelu_shift);
+    u.pc = (p.round_mode == NCE_ROUND_HALF_UP && p.prelu_shift > 0) ? 0.5 : 0.0;
+    u.lo = p.lo;
+    u.hi = p.hi;
+    u.zp = p.zp_out;
+    u.even = p.round_mode == NCE_ROUND_HALF_EVEN;
+    u.sat = may_saturate;
+    u.prelu = !(p.prelu_mult == 1 && p.prelu_shift == 0);
+    const int64_t am = p.prelu_mult < 0 ? -(int64_t)p.prelu_mult : (int64_t)p.prelu_mult;
+    u.prelu_sat = am > ((int64_t)1 << p.prelu_shift);
+    return u;
+}
+
+__device__ __forceinline__ double clamp_i32_range(double v) {
+    return __builtin_fmin(__builtin_fmax(v, -2147483648.0), 2147483647.0);
+}
+
+// v = acc * M + B already formed by the caller (so that callers can fold more terms into it).
+__device__ __forceinline__ int32_t ppe_finish_f64(double v, const PpeF64& u) {
+    v = u.even ? __builtin_rint(v) : __builtin_floor(v);
+    if (u.sat) v = clamp_i32_range(v);
+    if (u.prelu) {
+        double r = __builtin_fma(v, u.pm, u.pc);
+        r = u.even ? __builtin_rint(r) : __builtin_floor(r);
+        if (u.prelu_sat) r = clamp_i32_range(r);
+        v = v < 0.0 ? r : v;
+    }
+    int32_t y = (int32_t)v;  // in range by construction
+    y = y < u.lo ? u.lo : (y > u.hi ? u.hi : y);
+    return y + u.zp;
+}
+
+__device__ __forceinline__ int32_t ppe_apply_f64(int32_t acc, double M, double B, const PpeF64& u) {
+    return ppe_finish_f64(__builtin_fma((double)acc, M, B), u);
 }
 
 }  // namespace nce

@@ -7,8 +7,16 @@
 // Depthwise weights are one 16-byte-multiple row per channel holding the KY*KX taps row-major
 // (src/vpux_compiler/src/dialect/VPU/utils/const_utils.cpp:101-120,216-243).
 //
-// Memory-bound: a lane owns one 16-channel group (one 128-bit load per tap) of one output pixel;
-// adjacent lanes own adjacent channel groups, so a wavefront reads whole NHWC pixels contiguously.
+// Memory-bound kernels: a lane owns one 16-channel group (one 128-bit load per tap) of one output
+// pixel; adjacent lanes own adjacent channel groups, so a wavefront reads whole NHWC pixels
+// contiguously. Arithmetic is kept below the memory time:
+//   * sums run in FP32 on v_cvt_f32_ubyteN (byte -> float in one instruction) + v_fma_f32. Every
+//     partial sum is an integer below 2^24 (121 taps * 255 * 255), so FP32 is exact.
+//   * bytes are taken as unsigned (i8 storage is re-biased by x ^ 0x80) and out-of-image taps are
+//     filled with the zero point, so they contribute 0; the constant  -zp * sum(w)  is folded into
+//     the per-channel bias.
+//   * the requantize runs in FP64 (see nce_ppe_device.h); shifts above 52 take the integer path.
+//   * MAXPOOL compares two channels per instruction (even / odd bytes as packed u16).
 #include "nce_ppe_device.h"
 
 namespace nce {
@@ -16,36 +24,95 @@ namespace {
 
 enum { MODE_DW = 0, MODE_AVG = 1, MODE_MAX = 2 };
 
-constexpr int SLAB_GROUPS = 16;                  // channel groups (of 16) one block works on
-constexpr int SLAB_CH = SLAB_GROUPS * 16;        // 256 channels
+constexpr int SLAB_GROUPS = 8;             // channel groups (of 16) one block works on
+constexpr int SLAB_CH = SLAB_GROUPS * 16;  // 128 channels
+constexpr int NT = 256;
 
-template <bool SIGNED>
-__device__ __forceinline__ int32_t byte_at(uint32_t w, int i) {
-    return SIGNED ? (int32_t)(int8_t)(w >> (8 * i)) : (int32_t)((w >> (8 * i)) & 0xFFu);
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float ubyte_f32(uint32_t w, int i) {
+    // the compiler turns this into v_cvt_f32_ubyte{i}
+    return (float)((w >> (8 * i)) & 0xFFu);
 }
 
-template <int MODE, bool A_SIGNED, bool W_SIGNED>
-__global__ __launch_bounds__(256) void window_kernel(TaskDev t, Box box, int64_t npix, int items_per_thread) {
-    extern __shared__ uint8_t s_w[];  // MODE_DW: [tap][SLAB_CH] weight bytes of this block's channel slab
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    const u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b));
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    const u16x2 r = __builtin_elementwise_min(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b));
+    return __builtin_bit_cast(uint32_t, r);
+}
 
+struct WinArgs {
+    TaskDev t;
+    Box box;
+    int64_t npix;
+    int32_t items_per_thread;
+    uint32_t a_xor;   // 0x80808080 for i8 activations
+    uint32_t fill;    // word of re-biased zero-point bytes for out-of-image taps
+    int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
+};
+
+template <int MODE>
+__global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
+    // MODE_DW: [tap][SLAB_CH] floats of (w - zp_w); then per-channel FP64 scale constants
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ double sM[SLAB_CH], sB[SLAB_CH];
+    __shared__ int32_t sMult[SLAB_CH], sShift[SLAB_CH], sBias[SLAB_CH], sCorr[SLAB_CH];
+
+    const TaskDev& t = a.t;
+    const Box& box = a.box;
     const int32_t cgroups = box.bc >> 4;
-    const int32_t slab0 = blockIdx.y * SLAB_GROUPS;  // first channel group of the slab
+    const int32_t slab0 = blockIdx.y * SLAB_GROUPS;
     const int32_t nslab = min(SLAB_GROUPS, cgroups - slab0);
     const int ntaps = t.ky * t.kx;
+    float* s_w = reinterpret_cast<float*>(smem);
 
-    if (MODE == MODE_DW) {
-        // transpose [channel][tap] rows into [tap][channel]
-        for (int ch = threadIdx.x; ch < nslab * 16; ch += blockDim.x) {
-            const uint8_t* row = t.weights + (int64_t)(box.z0 + slab0 * 16 + ch) * t.w_stride_oc;
-            for (int tap = 0; tap < ntaps; ++tap) s_w[tap * SLAB_CH + ch] = row[tap];
+    // ---- per-channel constants ---------------------------------------------------------------
+    int bad_shift = 0, small_shift = 0;
+    if (MODE != MODE_MAX) {
+        for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
+            const int32_t c = box.z0 + slab0 * 16 + ch;
+            int32_t wsum = 0;
+            if (MODE == MODE_DW) {
+                const uint8_t* row = t.weights + (int64_t)c * t.w_stride_oc;
+                for (int tap = 0; tap < ntaps; ++tap) {
+                    const int32_t w = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
+                    wsum += w;
+                    s_w[tap * SLAB_CH + ch] = (float)w;
+                }
+            } else {
+                wsum = ntaps;
+            }
+            int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
+            if (t.table != nullptr) {
+                const int32_t* row = t.table + (int64_t)c * t.table_stride;
+                mult = table_mult(row[2]);
+                shift = table_shift(row[2]);
+                bias = row[3];
+            }
+            // out-of-image taps were filled with the zero point: remove zpu * sum(w) exactly
+            const int32_t corr = -a.zpu * wsum;
+            sMult[ch] = mult;
+            sShift[ch] = shift;
+            sBias[ch] = bias;
+            sCorr[ch] = corr;  // |corr| < 2^23
+            const double M = ppe_scale_M(mult, shift);
+            sM[ch] = M;
+            sB[ch] = __builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode));
+            bad_shift |= shift > kMaxF64Shift;
+            small_shift |= shift < kNoSatShift;
         }
-        __syncthreads();
     }
+    const bool use_int = __syncthreads_or(bad_shift) != 0;
+    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
 
-    const int64_t nitems = npix * nslab;
-    const int64_t first = (int64_t)blockIdx.x * blockDim.x * items_per_thread;
-    for (int it = 0; it < items_per_thread; ++it) {
-        const int64_t item = first + (int64_t)it * blockDim.x + threadIdx.x;
+    const int64_t nitems = a.npix * nslab;
+    const int64_t first = (int64_t)blockIdx.x * NT * a.items_per_thread;
+    for (int it = 0; it < a.items_per_thread; ++it) {
+        const int64_t item = first + (int64_t)it * NT + threadIdx.x;
         if (item >= nitems) break;
         const int32_t cg = (int32_t)(item % nslab);
         int64_t r = item / nslab;
@@ -57,79 +124,118 @@ __global__ __launch_bounds__(256) void window_kernel(TaskDev t, Box box, int64_t
         const int32_t oy = box.y0 + by, ox = box.x0 + bx;
         const int32_t iy0 = oy * t.sy - t.pt, ix0 = ox * t.sx - t.pl;
         const uint8_t* src = t.in.data + n * t.in.sn + oc;
+        uint8_t* dst = t.out.data + n * t.out.sn + (int64_t)oy * t.out.sh + (int64_t)ox * t.out.sw + oc;
 
-        int32_t acc[16];
-        const int32_t init = MODE == MODE_MAX ? (A_SIGNED ? -128 : 0) : 0;
+        if (MODE == MODE_MAX) {
+            // even / odd bytes of each dword as packed u16; order-preserving re-bias for i8
+            uint32_t me[4] = {0, 0, 0, 0}, mo[4] = {0, 0, 0, 0};
+            for (int ky = 0; ky < t.ky; ++ky) {
+                const int32_t iy = iy0 + ky;
+                if ((uint32_t)iy >= (uint32_t)t.in.h) continue;
+                for (int kx = 0; kx < t.kx; ++kx) {
+                    const int32_t ix = ix0 + kx;
+                    if ((uint32_t)ix >= (uint32_t)t.in.w) continue;
+                    const uint4 va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                    const uint32_t wa[4] = {va.x ^ a.a_xor, va.y ^ a.a_xor, va.z ^ a.a_xor, va.w ^ a.a_xor};
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = init;
+                    for (int d = 0; d < 4; ++d) {
+                        me[d] = pk_max_u16(me[d], wa[d] & 0x00FF00FFu);
+                        mo[d] = pk_max_u16(mo[d], (wa[d] >> 8) & 0x00FF00FFu);
+                    }
+                }
+            }
+            // clamp in the re-biased domain (lo/hi shifted by 128 for i8), then undo the re-bias
+            const uint32_t off = t.in.is_signed ? 128u : 0u;
+            const uint32_t lo2 = ((uint32_t)(t.ppe.lo + (int32_t)off)) * 0x00010001u;
+            const uint32_t hi2 = ((uint32_t)(t.ppe.hi + (int32_t)off)) * 0x00010001u;
+            uint32_t wo[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t e = pk_min_u16(pk_max_u16(me[d], lo2), hi2);
+                const uint32_t o = pk_min_u16(pk_max_u16(mo[d], lo2), hi2);
+                wo[d] = (e | (o << 8)) ^ a.a_xor;
+            }
+            *reinterpret_cast<uint4*>(dst) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+            continue;
+        }
 
+        float acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
         for (int ky = 0; ky < t.ky; ++ky) {
             const int32_t iy = iy0 + ky;
-            if (iy < 0 || iy >= t.in.h) continue;
+            const bool row_in = (uint32_t)iy < (uint32_t)t.in.h;
             for (int kx = 0; kx < t.kx; ++kx) {
                 const int32_t ix = ix0 + kx;
-                if (ix < 0 || ix >= t.in.w) continue;
-                const uint4 va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                uint4 va = make_uint4(a.fill, a.fill, a.fill, a.fill);
+                if (row_in && (uint32_t)ix < (uint32_t)t.in.w) {
+                    va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                    va.x ^= a.a_xor;
+                    va.y ^= a.a_xor;
+                    va.z ^= a.a_xor;
+                    va.w ^= a.a_xor;
+                }
                 const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
                 if (MODE == MODE_DW) {
-                    const uint4 vw = *reinterpret_cast<const uint4*>(s_w + (ky * t.kx + kx) * SLAB_CH + (cg << 4));
-                    const uint32_t ww[4] = {vw.x, vw.y, vw.z, vw.w};
+                    const float4* wp = reinterpret_cast<const float4*>(s_w + (ky * t.kx + kx) * SLAB_CH + (cg << 4));
 #pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        acc[i] += (byte_at<A_SIGNED>(wa[i >> 2], i & 3) - t.in.zp) *
-                                  (byte_at<W_SIGNED>(ww[i >> 2], i & 3) - t.w_zp);
-                } else if (MODE == MODE_AVG) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[i] += byte_at<A_SIGNED>(wa[i >> 2], i & 3) - t.in.zp;
+                    for (int d = 0; d < 4; ++d) {
+                        const float4 w4 = wp[d];
+                        acc[4 * d + 0] = __builtin_fmaf(ubyte_f32(wa[d], 0), w4.x, acc[4 * d + 0]);
+                        acc[4 * d + 1] = __builtin_fmaf(ubyte_f32(wa[d], 1), w4.y, acc[4 * d + 1]);
+                        acc[4 * d + 2] = __builtin_fmaf(ubyte_f32(wa[d], 2), w4.z, acc[4 * d + 2]);
+                        acc[4 * d + 3] = __builtin_fmaf(ubyte_f32(wa[d], 3), w4.w, acc[4 * d + 3]);
+                    }
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[i] = max(acc[i], byte_at<A_SIGNED>(wa[i >> 2], i & 3));
+                    for (int i = 0; i < 16; ++i) acc[i] += ubyte_f32(wa[i >> 2], i & 3);
                 }
             }
         }
 
         uint32_t wo[4] = {0, 0, 0, 0};
+        const int chl = cg << 4;
+        if (!use_int) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            int32_t y;
-            if (MODE == MODE_MAX) {
-                y = acc[i] < t.ppe.lo ? t.ppe.lo : (acc[i] > t.ppe.hi ? t.ppe.hi : acc[i]);
-            } else {
-                int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
-                if (t.table != nullptr) {
-                    const int32_t* row = t.table + (int64_t)(oc + i) * t.table_stride;
-                    mult = table_mult(row[2]);
-                    shift = table_shift(row[2]);
-                    bias = row[3];
-                }
-                y = ppe_apply(acc[i], bias, mult, shift, t.ppe);
+            for (int i = 0; i < 16; ++i) {
+                const int32_t y = ppe_finish_f64(__builtin_fma((double)acc[i], sM[chl + i], sB[chl + i]), pu);
+                wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
             }
-            wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                // acc + corr is the true accumulator (|.| < 2^23); the table bias is added in 64 bits inside
+                const int32_t y = ppe_apply((int32_t)acc[i] + sCorr[chl + i], sBias[chl + i], sMult[chl + i], sShift[chl + i], t.ppe);
+                wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
+            }
         }
-        *reinterpret_cast<uint4*>(t.out.data + n * t.out.sn + (int64_t)oy * t.out.sh + (int64_t)ox * t.out.sw + oc) =
-                make_uint4(wo[0], wo[1], wo[2], wo[3]);
+        *reinterpret_cast<uint4*>(dst) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
     }
 }
 
 template <int MODE>
 hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
-    const int64_t npix = (int64_t)t.out.n * box.bh * box.bw;
+    WinArgs a;
+    a.t = t;
+    a.box = box;
+    a.npix = (int64_t)t.out.n * box.bh * box.bw;
     const int32_t cgroups = box.bc >> 4;
-    if (npix == 0 || cgroups == 0) return hipSuccess;
+    if (a.npix == 0 || cgroups == 0) return hipSuccess;
     const int nslabs = (cgroups + SLAB_GROUPS - 1) / SLAB_GROUPS;
-    const int64_t items = npix * (cgroups < SLAB_GROUPS ? cgroups : SLAB_GROUPS);
-    const int ipt = items > (int64_t)256 * 4096 ? 4 : 1;
-    const int64_t blocks = (items + 256 * ipt - 1) / (256 * ipt);
+    const int64_t items = a.npix * (cgroups < SLAB_GROUPS ? cgroups : SLAB_GROUPS);
+    a.items_per_thread = items > (int64_t)NT * 8192 ? 4 : 1;
+    const int64_t blocks = (items + NT * a.items_per_thread - 1) / (NT * a.items_per_thread);
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    const size_t lds = MODE == MODE_DW ? (size_t)t.ky * t.kx * SLAB_CH : 0;
-    const dim3 grid((unsigned)blocks, (unsigned)nslabs);
-    const int sel = (t.in.is_signed ? 2 : 0) | (t.w_is_signed ? 1 : 0);
-    switch (sel) {
-    case 0: hipLaunchKernelGGL((window_kernel<MODE, false, false>), grid, dim3(256), lds, s, t, box, npix, ipt); break;
-    case 1: hipLaunchKernelGGL((window_kernel<MODE, false, true>), grid, dim3(256), lds, s, t, box, npix, ipt); break;
-    case 2: hipLaunchKernelGGL((window_kernel<MODE, true, false>), grid, dim3(256), lds, s, t, box, npix, ipt); break;
-    default: hipLaunchKernelGGL((window_kernel<MODE, true, true>), grid, dim3(256), lds, s, t, box, npix, ipt); break;
+    a.a_xor = t.in.is_signed ? 0x80808080u : 0u;
+    a.zpu = t.in.zp + (t.in.is_signed ? 128 : 0);
+    a.fill = (uint32_t)a.zpu * 0x01010101u;
+    const size_t lds = MODE == MODE_DW ? (size_t)t.ky * t.kx * SLAB_CH * sizeof(float) : 0;
+    if (lds > 32 * 1024) {  // large depthwise kernels: opt in to more than the default dynamic LDS
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&window_kernel<MODE>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
     }
+    hipLaunchKernelGGL((window_kernel<MODE>), dim3((unsigned)blocks, (unsigned)nslabs), dim3(NT), lds, s, a);
     return hipGetLastError();
 }
 

@@ -78,10 +78,19 @@ def test_conv_ppe_variants(executor, ppe):
     check(K.conv_case(21, 1, 12, 12, 32, 32, ppe=ppe), executor)
 
 
-@pytest.mark.parametrize("scale_lo,scale_hi", [(1e-6, 1e-5), (1e-2, 1e-1), (0.3, 0.9), (1.0, 7.9), (20.0, 255.0)])
+@pytest.mark.parametrize("scale_lo,scale_hi", [(1e-6, 1e-5), (1e-2, 1e-1), (0.3, 0.9), (1.0, 7.9), (20.0, 255.0),
+                                               (2e-13, 9e-13), (1e-12, 1e-3)])
 def test_conv_scale_ranges(executor, scale_lo, scale_hi):
     # small scales -> shift up to 34; large scales -> shift down to 7 and saturating outputs
     check(K.conv_case(33, 1, 8, 8, 32, 32, scale_lo=scale_lo, scale_hi=scale_hi), executor)
+
+
+@pytest.mark.parametrize("scale_lo,scale_hi", [(2e-13, 9e-13), (1e-12, 1e-3), (3.0, 200.0)])
+def test_dwconv_scale_ranges(executor, scale_lo, scale_hi):
+    # shifts above 52 take the integer epilogue, shifts below 18 the saturating one
+    check(K.dw_case(34, 1, 9, 9, 32, scale_lo=scale_lo, scale_hi=scale_hi), executor)
+    check(K.dw_case(35, 1, 9, 9, 32, scale_lo=scale_lo, scale_hi=scale_hi,
+                    ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=2047, lrelu_shift=0)), executor)
 
 
 def test_dwconv_cfg3_small(executor):
@@ -127,7 +136,10 @@ def test_eltwise_cfg4_small(executor):
                                 dict(ppe_extra=dict(round_mode=nce.ROUND_HALF_EVEN)),
                                 dict(ppe_extra=dict(mode=nce.PPE_LRELU, clamp_low=128)),
                                 dict(in1_mult=65535, in2_mult=65535, mult=65535, shift=40),
-                                dict(mult=3, shift=0, in1_mult=1, in2_mult=1)])
+                                dict(mult=3, shift=0, in1_mult=1, in2_mult=1),
+                                dict(mult=40000, shift=53), dict(mult=65535, shift=63),
+                                dict(mult=65535, shift=10, ppe_extra=dict(mode=nce.PPE_LPRELU, lrelu_mult=-2047, lrelu_shift=0)),
+                                dict(ppe_extra=dict(round_mode=nce.ROUND_NONE))])
 def test_eltwise_variants(executor, kw):
     check(K.eltwise_case(11, 1, 7, 9, 48, **kw), executor)
 
