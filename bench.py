@@ -83,6 +83,37 @@ def measure(ex, name, maker, bound, steps, warmup):
                   "bytes_per_step": nbytes, "roofline": roof}
 
 
+def measure_graph(ex, steps, warmup, batch=32):
+    """cfg5: the whole ResNet-50 task graph (53 convs + max pool + 16 adds) as one step."""
+    import torch
+    from npu_plugin_amd import workloads as W
+    graph = W.ResNet50Graph(batch=batch)
+    dg = W.DeviceGraph(graph, ex, graph.make_input())
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(max(1, warmup)):
+        dg.run(stream)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        dg.run(stream)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    ev = e0.elapsed_time(e1) * 1e-3 / steps
+    ops = graph.conv_ops()
+    conv_bytes = sum(graph.layer_bytes(L) for L in graph.layers if L.task_type == 0)
+    other_bytes = sum(graph.layer_bytes(L) for L in graph.layers if L.task_type != 0)
+    roof = {"bound": "mfma", "achieved": ops / ev / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+            "frac": ops / ev / 1e12 / PEAK_INT8_TOPS, "traffic": None, "kernel_us": ev * 1e6,
+            "note": "whole graph per step: 53 conv kernels + 1 max pool + 16 adds, launched back to back"}
+    dg.task_list.destroy()
+    return {"workload": f"cfg5_resnet50_b{batch}_224 (70 tasks)", "value": ops / wall / 1e9, "unit": "GOPS",
+            "ms_per_step": wall * 1e3, "ops_per_step": ops, "conv_bytes_per_step": conv_bytes,
+            "pool_add_bytes_per_step": other_bytes, "roofline": roof}
+
+
 def cpu_baseline(case, bound, budget_s=12.0):
     """The CPU oracle (a port of the reference's semantics; the reference itself has no executable
     arithmetic for this path) timed on the host cores, on whole passes of the same workload."""
@@ -153,6 +184,7 @@ def main():
                 continue
             _, r = measure(ex, name, mk, bd, args.steps, args.warmup)
             others[name] = r
+        others["cfg5"] = measure_graph(ex, max(5, args.steps // 10), max(2, args.warmup // 10))
         line["other_workloads"] = others
     ex.destroy()
     print(json.dumps(line))

@@ -259,3 +259,155 @@ def cfg3_avgpool(n=16, x=None):
 
 def cfg4(n=16):
     return eltwise_case(SEED + 6, n, 28, 28, 256, name=f"cfg4_eltwise_{n}x28x28x256")
+
+
+# ------------------------------------------------------------------------------------------------
+# cfg5: synthetic INT8 ResNet-50 (v1.5) chained through the NCE op path
+# ------------------------------------------------------------------------------------------------
+
+@dataclass
+class GraphLayer:
+    name: str
+    task_type: int
+    src: int                      # index of the input tensor in the graph's tensor list
+    src2: int = -1                # second input (eltwise)
+    dst: int = -1
+    weights: np.ndarray = None
+    table: np.ndarray = None
+    kernel: tuple = None
+    strides: tuple = None
+    pads: tuple = (0, 0, 0, 0)
+    ppe: dict = field(default_factory=dict)
+    real_ic: int = 0              # un-padded input channels (conv1), for the op count
+
+
+class ResNet50Graph:
+    """53 convolutions (1x1 / 3x3 / 7x7, strides 1 / 2), the 3x3 s2 max pool after conv1 and the 16
+    residual adds of ResNet-50 v1.5, all u8 NHWC with zero point 128, random i8 weights and random
+    per-channel mult/shift tables. ReLU is the 37XX form: mode NOOP, clamp [zp, 255]."""
+
+    ZP = 128
+
+    def __init__(self, batch=32, size=224, seed=SEED + 7):
+        self.batch, self.size = batch, size
+        self.rng = np.random.default_rng(seed)
+        self.tensors = []   # shapes (N, H, W, C)
+        self.layers = []
+        x = self._tensor(size, size, 16)      # 3 real channels padded to 16 (zero weights on the padding)
+        x = self._conv("conv1", x, 64, (7, 7), (2, 2), (3, 3, 3, 3), relu=True, real_ic=3)
+        x = self._maxpool("pool1", x)
+        inplanes = 64
+        for li, (planes, blocks, stride) in enumerate([(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)], 1):
+            for b in range(blocks):
+                s = stride if b == 0 else 1
+                name = f"layer{li}.{b}"
+                y = self._conv(name + ".conv1", x, planes, (1, 1), (1, 1), (0, 0, 0, 0), relu=True)
+                y = self._conv(name + ".conv2", y, planes, (3, 3), (s, s), (1, 1, 1, 1), relu=True)
+                y = self._conv(name + ".conv3", y, planes * 4, (1, 1), (1, 1), (0, 0, 0, 0), relu=False)
+                if b == 0:
+                    idt = self._conv(name + ".downsample", x, planes * 4, (1, 1), (s, s), (0, 0, 0, 0), relu=False)
+                else:
+                    idt = x
+                x = self._add(name + ".add", y, idt)
+                inplanes = planes * 4
+        self.output = x
+
+    # -- construction helpers --------------------------------------------------------------------
+    def _tensor(self, h, w, c):
+        self.tensors.append((self.batch, h, w, c))
+        return len(self.tensors) - 1
+
+    def _conv(self, name, src, oc, k, s, pads, relu, real_ic=0):
+        _, h, w, ic = self.tensors[src]
+        wt = self.rng.integers(-127, 128, size=(oc, k[0], k[1], ic), dtype=np.int64).astype(np.int8)
+        if real_ic:
+            wt[:, :, :, real_ic:] = 0
+        # Keep activations alive through 50 layers: aim every conv at a pre-activation spread of ~40
+        # quantization steps. Inputs are post-ReLU (rms ~ 40 / sqrt(2)) except the image (uniform bytes).
+        kk = k[0] * k[1] * (real_ic or ic)
+        in_rms = 73.9 if real_ic else 40.0 / math.sqrt(2.0)
+        base = 40.0 / (math.sqrt(kk) * in_rms * 73.3)
+        table = make_table(self.rng, oc, k[0] * k[1] * ic, 0.85 * base, 1.15 * base, bias_sigma=5.0 / base)
+        oh, ow = out_hw(h, w, k, s, pads)
+        dst = self._tensor(oh, ow, oc)
+        ppe = dict(mode=nce.PPE_NOOP, clamp_low=self.ZP if relu else 0, clamp_high=255)
+        self.layers.append(GraphLayer(name, nce.TASK_CONV, src, -1, dst, wt, table, tuple(k), tuple(s), tuple(pads), ppe,
+                                      real_ic or ic))
+        return dst
+
+    def _maxpool(self, name, src):
+        _, h, w, c = self.tensors[src]
+        oh, ow = out_hw(h, w, (3, 3), (2, 2), (1, 1, 1, 1))
+        dst = self._tensor(oh, ow, c)
+        self.layers.append(GraphLayer(name, nce.TASK_MAXPOOL, src, -1, dst, None, None, (3, 3), (2, 2), (1, 1, 1, 1),
+                                      dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255)))
+        return dst
+
+    def _add(self, name, a, b):
+        _, h, w, c = self.tensors[a]
+        dst = self._tensor(h, w, c)
+        # (a + b) / sqrt(2), ReLU: both inputs x 16384 (shift 14 folded into the output shift)
+        ppe = dict(mode=nce.PPE_NOOP, clamp_low=self.ZP, clamp_high=255, quant_mult=23170, quant_shift=29,
+                   in1_quant_mult=16384, in2_quant_mult=16384)
+        self.layers.append(GraphLayer(name, nce.TASK_ELTWISE, a, b, dst, None, None, None, None, (0, 0, 0, 0), ppe))
+        return dst
+
+    # -- accounting ------------------------------------------------------------------------------
+    def conv_ops(self):
+        total = 0
+        for L in self.layers:
+            if L.task_type == nce.TASK_CONV:
+                n, oh, ow, oc = self.tensors[L.dst]
+                total += 2 * n * oh * ow * oc * L.kernel[0] * L.kernel[1] * L.real_ic
+        return total
+
+    def layer_bytes(self, L):
+        b = int(np.prod(self.tensors[L.src])) + int(np.prod(self.tensors[L.dst]))
+        if L.src2 >= 0:
+            b += int(np.prod(self.tensors[L.src2]))
+        if L.weights is not None:
+            b += L.weights.nbytes + L.table.nbytes
+        return b
+
+    def make_input(self):
+        x = self.rng.integers(0, 256, size=self.tensors[0], dtype=np.int64).astype(np.uint8)
+        return x
+
+    # -- task construction over any buffers (numpy or torch) -----------------------------------
+    def layer_case(self, L):
+        """A Case view of one layer (tensors filled in by the caller)."""
+        return Case(L.name, L.task_type, np.empty(0, dtype=np.uint8), self.tensors[L.dst], self.ZP, self.ZP, False, None, 0,
+                    None, L.kernel, L.strides, L.pads, L.ppe, None)
+
+    def build_tasks(self, buffers, weights, tables):
+        """buffers[i]: activation tensor i; weights/tables[j]: operands of layer j (None where absent)."""
+        tasks = []
+        for j, L in enumerate(self.layers):
+            case = self.layer_case(L)
+            case.input = buffers[L.src]            # only shapes/strides/addresses are read
+            if L.task_type == nce.TASK_ELTWISE:
+                case.w_zp = self.ZP
+                tasks.append(build_task(case, buffers[L.src], buffers[L.src2], None, buffers[L.dst]))
+            else:
+                tasks.append(build_task(case, buffers[L.src], weights[j], tables[j], buffers[L.dst]))
+        return tasks
+
+
+class DeviceGraph:
+    """A ResNet50Graph resident on the GPU: activations, weights, tables and one task list."""
+
+    def __init__(self, graph, executor, x=None, device="cuda:0"):
+        import torch
+        self.graph = graph
+        self.buffers = [torch.zeros(s, dtype=torch.uint8, device=device) for s in graph.tensors]
+        if x is not None:
+            self.buffers[0].copy_(torch.from_numpy(x))
+        self.weights = [torch.from_numpy(L.weights).to(device) if L.weights is not None else None for L in graph.layers]
+        self.tables = [torch.from_numpy(L.table).to(device) if L.table is not None else None for L in graph.layers]
+        self.tasks = graph.build_tasks(self.buffers, self.weights, self.tables)
+        self.task_list = executor.task_list()
+        for t in self.tasks:
+            self.task_list.append(t)
+
+    def run(self, stream):
+        self.task_list.enqueue(stream)

@@ -13,3 +13,15 @@ def run_oracle(case, nthreads=0):
     return out
 
 
+
+
+def run_graph_oracle(graph, x, nthreads=0):
+    """Every activation tensor of a ResNet50Graph computed by the oracle (host numpy buffers)."""
+    from oracle import nce_oracle
+    buffers = [np.zeros(s, dtype=np.uint8) for s in graph.tensors]
+    buffers[0][...] = x
+    weights = [L.weights for L in graph.layers]
+    tables = [L.table for L in graph.layers]
+    for task in graph.build_tasks(buffers, weights, tables):
+        nce_oracle.run(task, nthreads)
+    return buffers

@@ -230,3 +230,25 @@ def test_task_list_chain(executor):
     executor.synchronize(stream)
     tl.destroy()
     assert np.array_equal(d3.output.cpu().numpy(), y3)
+
+
+# ---- cfg5: the ResNet-50 task graph ---------------------------------------------------------------
+
+@pytest.mark.parametrize("batch,size", [(1, 224), (3, 96)])
+def test_resnet50_graph_every_tensor(executor, batch, size):
+    """All 70 tasks (53 convs, max pool, 16 adds) chained on the GPU through one task list; every
+    intermediate tensor must equal the oracle's, not just the last one."""
+    import torch
+    graph = K.ResNet50Graph(batch=batch, size=size)
+    x = graph.make_input()
+    print(f"[case] resnet50 graph batch={batch} size={size}", flush=True)
+    want = K.run_graph_oracle(graph, x)
+    dg = K.DeviceGraph(graph, executor, x)
+    stream = torch.cuda.current_stream().cuda_stream
+    dg.run(stream)
+    executor.synchronize(stream)
+    for L in graph.layers:
+        got = dg.buffers[L.dst].cpu().numpy()
+        assert np.array_equal(got, want[L.dst]), f"{L.name}: {(got != want[L.dst]).sum()} bytes differ"
+    assert len(np.unique(want[graph.output])) > 100, "degenerate network output"
+    dg.task_list.destroy()
