@@ -329,6 +329,7 @@ nce_result_t make_plan(nce_log_s* log, const nce_cluster_task_desc_t* t, Plan* p
         d.sx = t->kernel_strides[1];
         d.pt = t->kernel_pad_top;
         d.pl = t->kernel_pad_left;
+        d.pr = t->kernel_pad_right;
     }
 
     const nce_tensor_t& w = t->weights;

@@ -44,7 +44,7 @@ struct TaskDev {
     int32_t w_is_signed, w_zp;
     const int32_t* table;    // weight table rows of 4 x int32, or nullptr
     int64_t table_stride;    // int32 elements between rows
-    int32_t ky, kx, sy, sx, pt, pl;
+    int32_t ky, kx, sy, sx, pt, pl, pr;
     PpeDev ppe;
 };
 

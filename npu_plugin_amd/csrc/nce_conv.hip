@@ -13,48 +13,14 @@
 // difference between 128 and the real zero point is restored exactly in the epilogue:
 //   sum (a-zpa)(w-zpw) = sum a'w' + da * sum w' + dw * (sum a' + K*da),  a' = a-offa, da = offa-zpa ...
 // Out-of-image taps are filled with the byte zp_a, so that (a' + da) = 0 there.
-#include "nce_ppe_device.h"
+#include "nce_conv_common.h"
 
 namespace nce {
 namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
 constexpr int BN = 64;    // output channels per workgroup
 constexpr int ROW = 80;   // LDS row pitch: 64 bytes of K + 16 bytes of padding against bank conflicts
 constexpr int NTHREADS = 256;
-
-struct ConvArgs {
-    const uint8_t* in;
-    int64_t in_sn, in_sh, in_sw;
-    int32_t H, W;
-    const uint8_t* w;
-    int64_t w_soc;
-    const int32_t* table;
-    int64_t table_stride;
-    uint8_t* out;
-    int64_t out_sn, out_sh, out_sw;
-    int32_t x0, y0, z0, bw, bh, bc;
-    int64_t M;  // pixels in the box over all batches
-    int32_t KY, KX, SY, SX, PT, PL;
-    int32_t KG;   // 16-byte groups along K: KY*KX*IC/16
-    int32_t ICG;  // 16-byte groups per tap: IC/16
-    uint32_t a_xor, w_xor;  // 0x80808080 for u8 storage, 0 for i8
-    uint32_t fill;          // out-of-image activation word, re-biased
-    int32_t da, dw;         // (storage offset - zero point) of activations / weights
-    int32_t ktot;           // KY*KX*IC
-    PpeDev ppe;
-};
-
-__device__ __forceinline__ int32_t bytesum(uint4 v) {
-    int32_t s = 0;
-    s = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, s, false);
-    s = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, s, false);
-    s = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, s, false);
-    s = __builtin_amdgcn_sdot4((int)v.w, 0x01010101, s, false);
-    return s;
-}
 
 // PXF = 32-pixel fragments per wavefront; the workgroup tile is (4 * 32 * PXF) pixels x 64 channels.
 template <int PXF>
@@ -67,6 +33,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
     __shared__ int32_t sW2[BN], sBias[BN], sWsum[BN], sCorr[BN];
     __shared__ double sM[BN], sBc[BN];
     __shared__ int32_t sAsum[BM];
+    const EpiSmem es = {sM, sBc, sW2, sBias, sCorr, sWsum};
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -78,17 +45,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
     const int32_t oc0 = a.z0 + blockIdx.y * BN;
     const int32_t noc = min(BN, a.z0 + a.bc - oc0);
 
-    if (tid < BN) {
-        int32_t w2 = 0, b = 0;
-        if (tid < noc) {
-            const int32_t* row = a.table + (int64_t)(oc0 + tid) * a.table_stride;
-            w2 = row[2];
-            b = row[3];
-        }
-        sW2[tid] = w2;
-        sBias[tid] = b;
-        sWsum[tid] = 0;
-    }
+    epi_load_table(a, es, tid, NTHREADS, BN, oc0, noc);
     for (int i = tid; i < BM; i += NTHREADS) sAsum[i] = 0;
 
     // ---- staging assignment: thread -> (row, 16-byte group) -------------------------------
@@ -194,7 +151,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
 
     // MFMA row i of the weight operand carries channel 16*((i>>2)&1) + 4*(i>>3) + (i&3), so that the
     // 16 accumulator registers of a lane are 16 CONSECUTIVE channels (16*half .. 16*half+15).
-    const int a_row = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+    const int a_row = chan_of_row(l32);
     const int b_row0 = wave * 32 * PXF + l32;
 
     const int nsteps = (a.KG + 3) >> 2;
@@ -234,20 +191,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         }
         __syncthreads();
     }
-    int bad_shift = 0, small_shift = 0;
-    if (tid < BN) {
-        const int32_t w2 = sW2[tid];
-        const int32_t mult = table_mult(w2), shift = table_shift(w2);
-        const int32_t corr = a.da * sWsum[tid];  // |da| <= 255, |sum w'| < 2^23
-        const double M = ppe_scale_M(mult, shift);
-        sM[tid] = M;
-        sBc[tid] = __builtin_fma((double)corr, M, ppe_scale_B(sBias[tid], M, shift, a.ppe.round_mode));
-        sCorr[tid] = corr;
-        bad_shift = shift > kMaxF64Shift;
-        small_shift = shift < kNoSatShift;
-    }
-    const bool use_int = __syncthreads_or(bad_shift) != 0;
-    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    bool use_int, may_sat;
+    epi_constants(a, es, tid, NTHREADS, BN, &use_int, &may_sat);
     const PpeF64 pu = ppe_f64_setup(a.ppe, may_sat);
 
     // ---- PPE + store -----------------------------------------------------------------------------
@@ -267,44 +212,25 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
         a_corr[x] = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
     }
-#pragma unroll
-    for (int f = 0; f < 2; ++f) {
-        const int ocl = 32 * f + 16 * half;
-        if (ocl >= noc) continue;
-        uint32_t wo[PXF][4];
-#pragma unroll
-        for (int x = 0; x < PXF; ++x) wo[x][0] = wo[x][1] = wo[x][2] = wo[x][3] = 0;
-        if (!use_int) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const double M = sM[ocl + v], B = sBc[ocl + v];
-#pragma unroll
-                for (int x = 0; x < PXF; ++x) {
-                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)a_corr[x]);
-                    const int32_t y = ppe_apply_f64(av, M, B, pu);
-                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
-                }
-            }
-        } else {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int c = ocl + v;
-                const int32_t w2 = sW2[c];
-#pragma unroll
-                for (int x = 0; x < PXF; ++x) {
-                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)a_corr[x] + (uint32_t)sCorr[c]);
-                    const int32_t y = ppe_apply(av, sBias[c], table_mult(w2), table_shift(w2), a.ppe);
-                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
-                }
-            }
-        }
-#pragma unroll
-        for (int x = 0; x < PXF; ++x)
-            if (p_valid[x]) *reinterpret_cast<uint4*>(dst[x] + ocl) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
-    }
+    epi_store<2, PXF>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, use_int, pu);
 }
 
 }  // namespace
+
+hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream) {
+    const unsigned gy = (unsigned)((a.bc + BN - 1) / BN);
+    // Tile 256 pixels per workgroup only when that still leaves at least two workgroups per CU.
+    const int64_t wg256 = ((a.M + 255) / 256) * gy;
+    if (wg256 >= 512) {
+        const int64_t gx = (a.M + 255) / 256;
+        if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+    } else {
+        const int64_t gx = (a.M + 127) / 128;
+        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+    }
+    return hipGetLastError();
+}
 
 hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     ConvArgs a;
@@ -314,6 +240,7 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.in_sw = t.in.sw;
     a.H = t.in.h;
     a.W = t.in.w;
+    a.IC = t.in.c;
     a.w = t.weights;
     a.w_soc = t.w_stride_oc;
     a.table = t.table;
@@ -346,21 +273,13 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.dw = off_w - t.w_zp;
     const uint32_t fb = (uint32_t)((t.in.zp - off_a) & 0xFF);
     a.fill = fb * 0x01010101u;
+    a.pitchpx = t.in.w + t.pl + t.pr;
+    a.nslots_max = a.rows_max = a.nchunks = a.halo_bytes = 0;
     a.ppe = t.ppe;
     if (a.M == 0 || box.bc == 0) return hipSuccess;
-
-    const unsigned gy = (unsigned)((box.bc + BN - 1) / BN);
-    // Tile 256 pixels per workgroup only when that still leaves at least two workgroups per CU.
-    const int64_t wg256 = ((a.M + 255) / 256) * gy;
-    if (wg256 >= 512) {
-        const int64_t gx = (a.M + 255) / 256;
-        if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
-    } else {
-        const int64_t gx = (a.M + 127) / 128;
-        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
-    }
-    return hipGetLastError();
+    const hipError_t e = launch_conv_halo(a, stream);
+    if (e != hipErrorNotSupported) return e;
+    return launch_conv_gather(a, stream);
 }
 
 }  // namespace nce

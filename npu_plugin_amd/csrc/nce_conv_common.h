@@ -1,0 +1,154 @@
+// Shared pieces of the CONV kernels: launch arguments, MFMA operand types and the fused PPE store.
+#pragma once
+
+#include "nce_ppe_device.h"
+
+namespace nce {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct ConvArgs {
+    const uint8_t* in;
+    int64_t in_sn, in_sh, in_sw;
+    int32_t H, W, IC;
+    const uint8_t* w;
+    int64_t w_soc;
+    const int32_t* table;
+    int64_t table_stride;
+    uint8_t* out;
+    int64_t out_sn, out_sh, out_sw;
+    int32_t x0, y0, z0, bw, bh, bc;
+    int64_t M;  // pixels in the box over all batches
+    int32_t KY, KX, SY, SX, PT, PL;
+    int32_t KG;   // 16-byte groups along K: KY*KX*IC/16
+    int32_t ICG;  // 16-byte groups per tap: IC/16
+    uint32_t a_xor, w_xor;  // 0x80808080 for u8 storage, 0 for i8
+    uint32_t fill;          // out-of-image activation word, re-biased
+    int32_t da, dw;         // (storage offset - zero point) of activations / weights
+    int32_t ktot;           // KY*KX*IC
+    // halo kernel only
+    int32_t pitchpx;     // staged pixels per input row: W + pad_left + pad_right
+    int32_t nslots_max;  // input rows one tile may stage
+    int32_t rows_max;    // output rows one tile may touch
+    int32_t nchunks;     // 64-byte chunks along IC
+    int32_t halo_bytes;  // nslots_max * pitchpx * 64
+    PpeDev ppe;
+};
+
+__device__ __forceinline__ int32_t bytesum(uint4 v) {
+    int32_t s = 0;
+    s = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.w, 0x01010101, s, false);
+    return s;
+}
+
+// MFMA row i of the weight operand carries channel chan_of_row(i) of its 32-channel fragment, so
+// that the 16 accumulator registers of a lane (rows 8*(v/4) + 4*half + v%4) are 16 CONSECUTIVE
+// channels 16*half .. 16*half+15 and one 128-bit store writes them.
+__device__ __forceinline__ int chan_of_row(int i) {
+    return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
+}
+__device__ __forceinline__ int row_of_chan(int c) {
+    return 8 * ((c >> 2) & 3) + 4 * (c >> 4) + (c & 3);
+}
+
+// Per-channel epilogue constants in LDS (BN entries each).
+struct EpiSmem {
+    double* M;
+    double* B;
+    int32_t* w2;
+    int32_t* bias;
+    int32_t* corr;
+    int32_t* wsum;
+};
+
+// Load the weight-table rows of this workgroup's channels. Call before the main loop (all threads).
+__device__ __forceinline__ void epi_load_table(const ConvArgs& a, const EpiSmem& s, int tid, int nthreads, int bn,
+                                               int32_t oc0, int32_t noc) {
+    for (int c = tid; c < bn; c += nthreads) {
+        int32_t w2 = 0, b = 0;
+        if (c < noc) {
+            const int32_t* row = a.table + (int64_t)(oc0 + c) * a.table_stride;
+            w2 = row[2];
+            b = row[3];
+        }
+        s.w2[c] = w2;
+        s.bias[c] = b;
+        s.wsum[c] = 0;
+    }
+}
+
+// After the main loop (wsum complete, behind a barrier): FP64 constants per channel. Returns, for
+// the whole workgroup, whether the integer path must be used and whether int32 saturation can occur.
+__device__ __forceinline__ void epi_constants(const ConvArgs& a, const EpiSmem& s, int tid, int nthreads, int bn,
+                                              bool* use_int, bool* may_sat) {
+    int bad_shift = 0, small_shift = 0;
+    for (int c = tid; c < bn; c += nthreads) {
+        const int32_t w2 = s.w2[c];
+        const int32_t mult = table_mult(w2), shift = table_shift(w2);
+        const int32_t corr = a.da * s.wsum[c];  // |da| <= 255, |sum w'| < 2^23
+        const double M = ppe_scale_M(mult, shift);
+        s.M[c] = M;
+        s.B[c] = __builtin_fma((double)corr, M, ppe_scale_B(s.bias[c], M, shift, a.ppe.round_mode));
+        s.corr[c] = corr;
+        bad_shift |= shift > kMaxF64Shift;
+        small_shift |= shift < kNoSatShift;
+    }
+    *use_int = __syncthreads_or(bad_shift) != 0;
+    *may_sat = __syncthreads_or(small_shift) != 0;
+}
+
+// PPE + store of one wavefront's accumulators: AF channel fragments x BF pixel fragments.
+//   ocw     first channel (workgroup-local) of this wave's fragment 0
+//   dst[x]  output address of this lane's pixel of fragment x at workgroup channel 0 (valid[x] says
+//           whether that pixel exists)
+//   acorr   per-pixel accumulator correction (weights zero point), 0 when unused
+template <int AF, int BF>
+__device__ __forceinline__ void epi_store(const ConvArgs& a, const EpiSmem& s, v16i (&acc)[AF][BF], int ocw, int noc,
+                                          int half, uint8_t* const (&dst)[BF], const bool (&valid)[BF],
+                                          const int32_t (&acorr)[BF], bool use_int, const PpeF64& pu) {
+#pragma unroll
+    for (int f = 0; f < AF; ++f) {
+        const int ocl = ocw + 32 * f + 16 * half;
+        if (ocl >= noc) continue;
+        uint32_t wo[BF][4];
+#pragma unroll
+        for (int x = 0; x < BF; ++x) wo[x][0] = wo[x][1] = wo[x][2] = wo[x][3] = 0;
+        if (!use_int) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const double M = s.M[ocl + v], B = s.B[ocl + v];
+#pragma unroll
+                for (int x = 0; x < BF; ++x) {
+                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)acorr[x]);
+                    const int32_t y = ppe_apply_f64(av, M, B, pu);
+                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int c = ocl + v;
+                const int32_t w2 = s.w2[c];
+#pragma unroll
+                for (int x = 0; x < BF; ++x) {
+                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)acorr[x] + (uint32_t)s.corr[c]);
+                    const int32_t y = ppe_apply(av, s.bias[c], table_mult(w2), table_shift(w2), a.ppe);
+                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
+                }
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < BF; ++x)
+            if (valid[x]) *reinterpret_cast<uint4*>(dst[x] + ocl) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
+    }
+}
+
+hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream);
+// Returns hipErrorNotSupported when the shape does not fit the halo kernel (caller falls back).
+hipError_t launch_conv_halo(const ConvArgs& a, hipStream_t stream);
+
+}  // namespace nce

@@ -252,3 +252,52 @@ def test_resnet50_graph_every_tensor(executor, batch, size):
         assert np.array_equal(got, want[L.dst]), f"{L.name}: {(got != want[L.dst]).sum()} bytes differ"
     assert len(np.unique(want[graph.output])) > 100, "degenerate network output"
     dg.task_list.destroy()
+
+
+# ---- halo-staged conv kernel: every tile configuration, image-crossing tiles, partial slices -----
+
+HALO_CASES = [
+    # (n, h, w, ic, oc, k, s, pads)                      which tile the dispatcher picks
+    (8, 128, 128, 64, 128, (3, 3), (1, 1), (1, 1, 1, 1)),   # 128 ch x 256 px
+    (4, 128, 128, 64, 128, (3, 3), (1, 1), (1, 1, 1, 1)),   # 64 ch x 256 px
+    (1, 128, 128, 64, 128, (3, 3), (1, 1), (1, 1, 1, 1)),   # 64 ch x 128 px
+    (8, 56, 56, 64, 64, (3, 3), (1, 1), (1, 1, 1, 1)),      # 64 ch x 64 px (cfg2 shape)
+    (8, 128, 128, 128, 256, (1, 1), (1, 1), (0, 0, 0, 0)),  # 1x1, big tile
+    (2, 56, 56, 256, 64, (1, 1), (1, 1), (0, 0, 0, 0)),     # 1x1, deep K
+    (2, 56, 56, 256, 512, (1, 1), (2, 2), (0, 0, 0, 0)),    # 1x1 stride 2 (downsample)
+    (3, 56, 56, 128, 128, (3, 3), (2, 2), (1, 1, 1, 1)),    # 3x3 stride 2
+    (40, 7, 7, 512, 128, (3, 3), (1, 1), (1, 1, 1, 1)),     # tiles span several whole images
+    (9, 14, 14, 256, 256, (3, 3), (1, 1), (1, 1, 1, 1)),    # tiles cross image boundaries mid-row
+    (2, 30, 30, 96, 80, (3, 3), (1, 1), (1, 1, 1, 1)),      # partial 64-channel slice, ragged channels
+    (2, 30, 30, 160, 48, (1, 1), (1, 1), (0, 0, 0, 0)),
+    (2, 31, 29, 64, 64, (3, 3), (1, 2), (0, 1, 1, 0)),      # asymmetric stride and padding
+    (2, 20, 20, 64, 64, (5, 3), (1, 1), (1, 1, 2, 2)),      # tall kernel
+    (2, 20, 20, 64, 64, (1, 3), (1, 1), (1, 1, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("shape", HALO_CASES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}s{s[6][0]}")
+def test_conv_halo_kernel_shapes(executor, shape):
+    n, h, w, ic, oc, k, s, pads = shape
+    check(K.conv_case(200 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads,
+                      ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14)), executor)
+
+
+def test_conv_halo_zero_points_and_types(executor):
+    check(K.conv_case(301, 2, 20, 20, 64, 64, in_zp=3, out_zp=17), executor)                      # weight-sum correction
+    check(K.conv_case(302, 2, 20, 20, 128, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128), executor)
+    check(K.conv_case(303, 2, 20, 20, 64, 64, w_signed=False, w_zp=128, in_zp=121), executor)
+    check(K.conv_case(304, 2, 20, 20, 64, 64, w_signed=False, w_zp=127, in_zp=121), executor)      # falls back to the gather kernel
+
+
+def test_conv_halo_variants(executor):
+    full = K.conv_case(305, 2, 24, 20, 64, 128)
+    want = K.run_oracle(full)
+    tiled = K.conv_case(305, 2, 24, 20, 64, 128, variants=[((0, 0, 0), (19, 11, 63)), ((0, 12, 0), (19, 23, 63)),
+                                                           ((0, 0, 64), (9, 23, 127)), ((10, 0, 64), (19, 23, 127))])
+    assert np.array_equal(K.run_hip(tiled, executor), want)
+    part = K.conv_case(305, 2, 24, 20, 64, 128, variants=[((3, 5, 64), (17, 20, 127))])
+    canvas = np.full(part.out_shape, 0x5A, dtype=np.uint8)
+    from oracle import nce_oracle
+    nce_oracle.run(K.build_task(part, part.input, part.weights, part.table, canvas))
+    assert np.array_equal(K.run_hip(part, executor), canvas)
