@@ -191,9 +191,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         }
         __syncthreads();
     }
-    bool use_int, may_sat;
-    epi_constants(a, es, tid, NTHREADS, BN, &use_int, &may_sat);
-    const PpeF64 pu = ppe_f64_setup(a.ppe, may_sat);
+    PpeF64 pu;
+    const int mode = epi_constants(a, es, tid, NTHREADS, BN, &pu);
 
     // ---- PPE + store -----------------------------------------------------------------------------
     uint8_t* dst[PXF];
@@ -212,7 +211,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
         a_corr[x] = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
     }
-    epi_store<2, PXF>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, use_int, pu);
+    if (a.dw != 0) epi_store<2, PXF, true>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, mode, pu);
+    else epi_store<2, PXF, false>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, mode, pu);
 }
 
 }  // namespace

@@ -81,70 +81,88 @@ __device__ __forceinline__ void epi_load_table(const ConvArgs& a, const EpiSmem&
     }
 }
 
-// After the main loop (wsum complete, behind a barrier): FP64 constants per channel. Returns, for
-// the whole workgroup, whether the integer path must be used and whether int32 saturation can occur.
-__device__ __forceinline__ void epi_constants(const ConvArgs& a, const EpiSmem& s, int tid, int nthreads, int bn,
-                                              bool* use_int, bool* may_sat) {
+// After the main loop (wsum complete, behind a barrier): FP64 constants per channel and the PPE
+// specialisation the whole workgroup runs.
+__device__ __forceinline__ int epi_constants(const ConvArgs& a, const EpiSmem& s, int tid, int nthreads, int bn,
+                                             PpeF64* pu) {
     int bad_shift = 0, small_shift = 0;
+    for (int c = tid; c < bn; c += nthreads) {
+        const int32_t w2 = s.w2[c];
+        const int32_t shift = table_shift(w2);
+        bad_shift |= shift > kMaxF64Shift;
+        small_shift |= shift < kNoSatShift;
+    }
+    const bool use_int = __syncthreads_or(bad_shift) != 0;
+    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    *pu = ppe_f64_setup(a.ppe, may_sat);
+    const int mode = ppe_mode_of(*pu, use_int);
     for (int c = tid; c < bn; c += nthreads) {
         const int32_t w2 = s.w2[c];
         const int32_t mult = table_mult(w2), shift = table_shift(w2);
         const int32_t corr = a.da * s.wsum[c];  // |da| <= 255, |sum w'| < 2^23
         const double M = ppe_scale_M(mult, shift);
         s.M[c] = M;
-        s.B[c] = __builtin_fma((double)corr, M, ppe_scale_B(s.bias[c], M, shift, a.ppe.round_mode));
+        s.B[c] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(s.bias[c], M, shift, a.ppe.round_mode)), mode, *pu);
         s.corr[c] = corr;
-        bad_shift |= shift > kMaxF64Shift;
-        small_shift |= shift < kNoSatShift;
     }
-    *use_int = __syncthreads_or(bad_shift) != 0;
-    *may_sat = __syncthreads_or(small_shift) != 0;
+    __syncthreads();
+    return mode;
 }
 
 // PPE + store of one wavefront's accumulators: AF channel fragments x BF pixel fragments.
 //   ocw     first channel (workgroup-local) of this wave's fragment 0
 //   dst[x]  output address of this lane's pixel of fragment x at workgroup channel 0 (valid[x] says
 //           whether that pixel exists)
-//   acorr   per-pixel accumulator correction (weights zero point), 0 when unused
-template <int AF, int BF>
-__device__ __forceinline__ void epi_store(const ConvArgs& a, const EpiSmem& s, v16i (&acc)[AF][BF], int ocw, int noc,
-                                          int half, uint8_t* const (&dst)[BF], const bool (&valid)[BF],
-                                          const int32_t (&acorr)[BF], bool use_int, const PpeF64& pu) {
+//   acorr   per-pixel accumulator correction (weights zero point); ACORR = false: not used
+template <int AF, int BF, int MODE, bool ACORR>
+__device__ __forceinline__ void epi_store_mode(const ConvArgs& a, const EpiSmem& s, v16i (&acc)[AF][BF], int ocw, int noc,
+                                               int half, uint8_t* const (&dst)[BF], const bool (&valid)[BF],
+                                               const int32_t (&acorr)[BF], const PpeF64& pu) {
 #pragma unroll
     for (int f = 0; f < AF; ++f) {
         const int ocl = ocw + 32 * f + 16 * half;
         if (ocl >= noc) continue;
         uint32_t wo[BF][4];
 #pragma unroll
-        for (int x = 0; x < BF; ++x) wo[x][0] = wo[x][1] = wo[x][2] = wo[x][3] = 0;
-        if (!use_int) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const double M = s.M[ocl + v], B = s.B[ocl + v];
-#pragma unroll
-                for (int x = 0; x < BF; ++x) {
-                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)acorr[x]);
-                    const int32_t y = ppe_apply_f64(av, M, B, pu);
-                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
-                }
+        for (int v = 0; v < 16; ++v) {
+            const int c = ocl + v;
+            double M = 0.0, B = 0.0;
+            int32_t w2 = 0, bias = 0, corr = 0;
+            if (MODE == PPE_MODE_INT) {
+                w2 = s.w2[c];
+                bias = s.bias[c];
+                corr = s.corr[c];
+            } else {
+                M = s.M[c];
+                B = s.B[c];
             }
-        } else {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int c = ocl + v;
-                const int32_t w2 = s.w2[c];
-#pragma unroll
-                for (int x = 0; x < BF; ++x) {
-                    const int32_t av = (int32_t)((uint32_t)acc[f][x][v] + (uint32_t)acorr[x] + (uint32_t)s.corr[c]);
-                    const int32_t y = ppe_apply(av, s.bias[c], table_mult(w2), table_shift(w2), a.ppe);
-                    wo[x][v >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (v & 3));
-                }
+            for (int x = 0; x < BF; ++x) {
+                int32_t av = acc[f][x][v];
+                if (ACORR) av = (int32_t)((uint32_t)av + (uint32_t)acorr[x]);
+                int32_t y;
+                if (MODE == PPE_MODE_INT)
+                    y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
+                else
+                    y = ppe_finish_mode<MODE>(__builtin_fma((double)av, M, B), pu);
+                const uint32_t b = (uint32_t)y & 0xFFu;
+                wo[x][v >> 2] = (v & 3) == 0 ? b : (wo[x][v >> 2] | (b << (8 * (v & 3))));
             }
         }
 #pragma unroll
         for (int x = 0; x < BF; ++x)
             if (valid[x]) *reinterpret_cast<uint4*>(dst[x] + ocl) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
     }
+}
+
+template <int AF, int BF, bool ACORR>
+__device__ __forceinline__ void epi_store(const ConvArgs& a, const EpiSmem& s, v16i (&acc)[AF][BF], int ocw, int noc,
+                                          int half, uint8_t* const (&dst)[BF], const bool (&valid)[BF],
+                                          const int32_t (&acorr)[BF], int mode, const PpeF64& pu) {
+    if (mode == PPE_MODE_FOLDED) epi_store_mode<AF, BF, PPE_MODE_FOLDED, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
+    else if (mode == PPE_MODE_SLOPE) epi_store_mode<AF, BF, PPE_MODE_SLOPE, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
+    else if (mode == PPE_MODE_ANY_F64) epi_store_mode<AF, BF, PPE_MODE_ANY_F64, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
+    else epi_store_mode<AF, BF, PPE_MODE_INT, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
 }
 
 hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream);

@@ -247,9 +247,8 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     }
 
     // ---- PPE + store --------------------------------------------------------------------------
-    bool use_int, may_sat;
-    epi_constants(a, es, tid, NT, BN, &use_int, &may_sat);
-    const PpeF64 pu = ppe_f64_setup(a.ppe, may_sat);
+    PpeF64 pu;
+    const int mode = epi_constants(a, es, tid, NT, BN, &pu);
     uint8_t* dst[BF];
     bool valid[BF];
     int32_t acorr[BF];
@@ -264,7 +263,7 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
         dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
         acorr[x] = 0;
     }
-    epi_store<AF, BF>(a, es, acc, wn * AF * 32, noc, half, dst, valid, acorr, use_int, pu);
+    epi_store<AF, BF, false>(a, es, acc, wn * AF * 32, noc, half, dst, valid, acorr, mode, pu);
 }
 
 // Exact staging bounds of a tiling: the largest number of output rows and of input-row slots any

@@ -25,7 +25,9 @@ struct EltArgs {
     int32_t may_sat;
 };
 
-// PATH 0: FP64 with uniform scale. PATH 1: integer, uniform scale. PATH 2: integer, per-channel table.
+// PATH = a PPE_MODE_* value with uniform scale, or PATH_TABLE: integer with a per-channel table.
+constexpr int PATH_TABLE = 4;
+
 template <bool FLAT, int PATH, bool SIGNED>
 __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
     const TaskDev& t = a.t;
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
         int32_t oc = 0;
         if (FLAT) {
             off_a = off_b = off_o = idx << 4;
-            if (PATH == 2) oc = (int32_t)(idx % cgroups) << 4;
+            if (PATH == PATH_TABLE) oc = (int32_t)(idx % cgroups) << 4;
         } else {
             int64_t r = idx;
             const int32_t cg = (int32_t)(r % cgroups);
@@ -66,15 +68,15 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
                 // |acc| < 2^26: 16-bit multipliers times 9-bit values, twice, plus c0
                 const int32_t acc = t.ppe.in1_mult * byte_at<SIGNED>(wa[d], i) + t.ppe.in2_mult * byte_at<SIGNED>(wb[d], i) + a.c0;
                 int32_t y;
-                if (PATH == 0) {
-                    y = ppe_apply_f64(acc, a.M, a.B, pu);
-                } else if (PATH == 1) {
+                if (PATH < PPE_MODE_INT) {
+                    y = ppe_finish_mode<PATH>(__builtin_fma((double)acc, a.M, a.B), pu);
+                } else if (PATH == PPE_MODE_INT) {
                     y = ppe_apply(acc, 0, t.ppe.quant_mult, t.ppe.quant_shift, t.ppe);
                 } else {
                     const int32_t* row = t.table + (int64_t)(oc + 4 * d + i) * t.table_stride;
                     y = ppe_apply(acc, row[3], table_mult(row[2]), table_shift(row[2]), t.ppe);
                 }
-                packed |= ((uint32_t)y & 0xFFu) << (8 * i);
+                packed = i == 0 ? ((uint32_t)y & 0xFFu) : (packed | (((uint32_t)y & 0xFFu) << (8 * i)));
             }
             wo[d] = packed;
         }
@@ -94,9 +96,11 @@ void launch_signed(const EltArgs& a, int grid, hipStream_t s) {
 
 template <bool FLAT>
 void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
-    if (path == 0) launch_signed<FLAT, 0>(a, grid, s);
-    else if (path == 1) launch_signed<FLAT, 1>(a, grid, s);
-    else launch_signed<FLAT, 2>(a, grid, s);
+    if (path == PPE_MODE_FOLDED) launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
+    else if (path == PPE_MODE_SLOPE) launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
+    else if (path == PPE_MODE_ANY_F64) launch_signed<FLAT, PPE_MODE_ANY_F64>(a, grid, s);
+    else if (path == PPE_MODE_INT) launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
+    else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
 
 }  // namespace
@@ -114,8 +118,19 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     const int shift = t.ppe.quant_shift;
     a.M = ldexp((double)t.ppe.quant_mult, -shift);
     a.B = (t.ppe.round_mode == NCE_ROUND_HALF_UP && shift > 0) ? 0.5 : 0.0;
-    a.may_sat = shift < 18;
-    const int path = t.table != nullptr ? 2 : (shift > 52 ? 1 : 0);
+    a.may_sat = shift < kNoSatShift;
+    // the same selection the table-driven kernels make per workgroup, made here on the host
+    const bool even = t.ppe.round_mode == NCE_ROUND_HALF_EVEN;
+    const bool prelu = !(t.ppe.prelu_mult == 1 && t.ppe.prelu_shift == 0);
+    const int64_t am = t.ppe.prelu_mult < 0 ? -(int64_t)t.ppe.prelu_mult : (int64_t)t.ppe.prelu_mult;
+    const bool prelu_sat = am > ((int64_t)1 << t.ppe.prelu_shift);
+    int path;
+    if (t.table != nullptr) path = PATH_TABLE;
+    else if (shift > kMaxF64Shift) path = PPE_MODE_INT;
+    else if (!even && !a.may_sat && !prelu) path = PPE_MODE_FOLDED;
+    else if (!even && !a.may_sat && prelu && !prelu_sat) path = PPE_MODE_SLOPE;
+    else path = PPE_MODE_ANY_F64;
+    if (path == PPE_MODE_FOLDED) a.B += (double)t.ppe.zp_out;
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (flat) launch_path<true>(a, path, (int)blocks, stream);

@@ -95,8 +95,47 @@ __device__ __forceinline__ double clamp_i32_range(double v) {
     return __builtin_fmin(__builtin_fmax(v, -2147483648.0), 2147483647.0);
 }
 
+// The wavefront-uniform flags are COMPILE-TIME here: a run-time flag inside the per-element code
+// makes the compiler evaluate both sides and select, which triples the instruction count.
 // v = acc * M + B already formed by the caller (so that callers can fold more terms into it).
-__device__ __forceinline__ int32_t ppe_finish_f64(double v, const PpeF64& u) {
+template <bool EVEN, bool SAT, bool PRELU, bool PSAT>
+__device__ __forceinline__ int32_t ppe_finish_f64_t(double v, const PpeF64& u) {
+    v = EVEN ? __builtin_rint(v) : __builtin_floor(v);
+    if (SAT) v = clamp_i32_range(v);
+    if (PRELU) {
+        double r = __builtin_fma(v, u.pm, u.pc);
+        r = EVEN ? __builtin_rint(r) : __builtin_floor(r);
+        if (PSAT) r = clamp_i32_range(r);
+        v = v < 0.0 ? r : v;
+    }
+    int32_t y = (int32_t)v;  // in range by construction
+    y = y < u.lo ? u.lo : (y > u.hi ? u.hi : y);
+    return y + u.zp;
+}
+
+// Fastest form: round half-up, no saturation, no slope, and the output zero point already folded into
+// B and into the clamp bounds (floor(x + zp) = floor(x) + zp for an integer zp).
+__device__ __forceinline__ int32_t ppe_finish_f64_folded(double v, int32_t lo_zp, int32_t hi_zp) {
+    const int32_t y = (int32_t)__builtin_floor(v);
+    return y < lo_zp ? lo_zp : (y > hi_zp ? hi_zp : y);
+}
+
+// Which specialisation a workgroup runs (uniform). 0: folded fast path, 1: half-up + slope,
+// 2: any flags (run-time selects), 3: integer arithmetic.
+enum { PPE_MODE_FOLDED = 0, PPE_MODE_SLOPE = 1, PPE_MODE_ANY_F64 = 2, PPE_MODE_INT = 3 };
+
+__device__ __forceinline__ int ppe_mode_of(const PpeF64& u, bool use_int) {
+    if (use_int) return PPE_MODE_INT;
+    if (!u.even && !u.sat && !u.prelu) return PPE_MODE_FOLDED;
+    if (!u.even && !u.sat && u.prelu && !u.prelu_sat) return PPE_MODE_SLOPE;
+    return PPE_MODE_ANY_F64;
+}
+
+template <int MODE>
+__device__ __forceinline__ int32_t ppe_finish_mode(double v, const PpeF64& u) {
+    if (MODE == PPE_MODE_FOLDED) return ppe_finish_f64_folded(v, u.lo + u.zp, u.hi + u.zp);
+    if (MODE == PPE_MODE_SLOPE) return ppe_finish_f64_t<false, false, true, false>(v, u);
+    // run-time flags
     v = u.even ? __builtin_rint(v) : __builtin_floor(v);
     if (u.sat) v = clamp_i32_range(v);
     if (u.prelu) {
@@ -105,13 +144,14 @@ __device__ __forceinline__ int32_t ppe_finish_f64(double v, const PpeF64& u) {
         if (u.prelu_sat) r = clamp_i32_range(r);
         v = v < 0.0 ? r : v;
     }
-    int32_t y = (int32_t)v;  // in range by construction
+    int32_t y = (int32_t)v;
     y = y < u.lo ? u.lo : (y > u.hi ? u.hi : y);
     return y + u.zp;
 }
 
-__device__ __forceinline__ int32_t ppe_apply_f64(int32_t acc, double M, double B, const PpeF64& u) {
-    return ppe_finish_f64(__builtin_fma((double)acc, M, B), u);
+// B constant of a channel for the given mode: the folded mode carries the output zero point.
+__device__ __forceinline__ double ppe_mode_B(double B, int mode, const PpeF64& u) {
+    return mode == PPE_MODE_FOLDED ? B + (double)u.zp : B;
 }
 
 }  // namespace nce

@@ -44,6 +44,18 @@ __device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// FP64 requantize of 16 channel sums with per-channel constants, packed into 4 dwords.
+template <int PMODE>
+__device__ __forceinline__ void requant16(const float (&acc)[16], const double* M, const double* B, const PpeF64& pu,
+                                          uint32_t (&wo)[4]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int32_t y = ppe_finish_mode<PMODE>(__builtin_fma((double)acc[i], M[i], B[i]), pu);
+        const uint32_t b = (uint32_t)y & 0xFFu;
+        wo[i >> 2] = (i & 3) == 0 ? b : (wo[i >> 2] | (b << (8 * (i & 3))));
+    }
+}
+
 struct WinArgs {
     TaskDev t;
     Box box;
@@ -70,7 +82,20 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     float* s_w = reinterpret_cast<float*>(smem);
 
     // ---- per-channel constants ---------------------------------------------------------------
+    // pass 1: which PPE specialisation the block runs (uniform); pass 2: the constants for it
     int bad_shift = 0, small_shift = 0;
+    if (MODE != MODE_MAX) {
+        for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
+            int32_t shift = t.ppe.quant_shift;
+            if (t.table != nullptr) shift = table_shift(t.table[(int64_t)(box.z0 + slab0 * 16 + ch) * t.table_stride + 2]);
+            bad_shift |= shift > kMaxF64Shift;
+            small_shift |= shift < kNoSatShift;
+        }
+    }
+    const bool use_int = __syncthreads_or(bad_shift) != 0;
+    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
+    const int pmode = ppe_mode_of(pu, use_int);
     if (MODE != MODE_MAX) {
         for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
             const int32_t c = box.z0 + slab0 * 16 + ch;
@@ -100,14 +125,10 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
             sCorr[ch] = corr;  // |corr| < 2^23
             const double M = ppe_scale_M(mult, shift);
             sM[ch] = M;
-            sB[ch] = __builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode));
-            bad_shift |= shift > kMaxF64Shift;
-            small_shift |= shift < kNoSatShift;
+            sB[ch] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu);
         }
     }
-    const bool use_int = __syncthreads_or(bad_shift) != 0;
-    const bool may_sat = __syncthreads_or(small_shift) != 0;
-    const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
+    __syncthreads();
 
     const int64_t nitems = a.npix * nslab;
     const int64_t first = (int64_t)blockIdx.x * NT * a.items_per_thread;
@@ -193,15 +214,13 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
             }
         }
 
-        uint32_t wo[4] = {0, 0, 0, 0};
+        uint32_t wo[4];
         const int chl = cg << 4;
-        if (!use_int) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int32_t y = ppe_finish_f64(__builtin_fma((double)acc[i], sM[chl + i], sB[chl + i]), pu);
-                wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
-            }
-        } else {
+        if (pmode == PPE_MODE_FOLDED) requant16<PPE_MODE_FOLDED>(acc, sM + chl, sB + chl, pu, wo);
+        else if (pmode == PPE_MODE_SLOPE) requant16<PPE_MODE_SLOPE>(acc, sM + chl, sB + chl, pu, wo);
+        else if (pmode == PPE_MODE_ANY_F64) requant16<PPE_MODE_ANY_F64>(acc, sM + chl, sB + chl, pu, wo);
+        else {
+            wo[0] = wo[1] = wo[2] = wo[3] = 0;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 // acc + corr is the true accumulator (|.| < 2^23); the table bias is added in 64 bits inside
