@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libnce_hip.so")
+# NCE_HIP_LIB points the loader at another build of the same library (kernel experiments).
+LIB_PATH = os.environ.get("NCE_HIP_LIB") or os.path.join(_HERE, "libnce_hip.so")
 
 # nce_result_t
 SUCCESS = 0

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
     const int half = lane >> 5;
     const int l32 = lane & 31;
 
-    const int64_t m0 = (int64_t)blockIdx.x * BM;
+    const int32_t m0 = blockIdx.x * BM;
     const int32_t oc0 = a.z0 + blockIdx.y * BN;
     const int32_t noc = min(BN, a.z0 + a.bc - oc0);
 
@@ -57,17 +57,16 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
     const uint8_t* b_base[NB];
     int32_t b_iy0[NB], b_ix0[NB];
     bool b_valid[NB];
-    const int64_t box_pix = (int64_t)a.bh * a.bw;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-        const int64_t p = m0 + srow + 64 * i;
+        const int32_t p = m0 + srow + 64 * i;
         b_valid[i] = p < a.M;
-        const int64_t pp = b_valid[i] ? p : 0;
-        const int64_t n = pp / box_pix;
-        const int32_t rem = (int32_t)(pp - n * box_pix);
-        const int32_t by = rem / a.bw;
-        const int32_t bx = rem - by * a.bw;
-        b_base[i] = a.in + n * a.in_sn;
+        const int32_t pp = b_valid[i] ? p : 0;
+        const int32_t rr = fdiv(pp, a.div_bw);
+        const int32_t bx = pp - rr * a.bw;
+        const int32_t n = fdiv(rr, a.div_bh);
+        const int32_t by = rr - n * a.bh;
+        b_base[i] = a.in + (int64_t)n * a.in_sn;
         b_iy0[i] = (a.y0 + by) * a.SY - a.PT;
         b_ix0[i] = (a.x0 + bx) * a.SX - a.PL;
     }
@@ -201,14 +200,14 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
 #pragma unroll
     for (int x = 0; x < PXF; ++x) {
         const int prow = b_row0 + 32 * x;
-        const int64_t p = m0 + prow;
+        const int32_t p = m0 + prow;
         p_valid[x] = p < a.M;
-        const int64_t pp = p_valid[x] ? p : 0;
-        const int64_t n = pp / box_pix;
-        const int32_t rem = (int32_t)(pp - n * box_pix);
-        const int32_t by = rem / a.bw;
-        const int32_t bx = rem - by * a.bw;
-        dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+        const int32_t pp = p_valid[x] ? p : 0;
+        const int32_t rr = fdiv(pp, a.div_bw);
+        const int32_t bx = pp - rr * a.bw;
+        const int32_t n = fdiv(rr, a.div_bh);
+        const int32_t by = rr - n * a.bh;
+        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
         a_corr[x] = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
     }
     if (a.dw != 0) epi_store<2, PXF, true>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, mode, pu);
@@ -220,13 +219,13 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
 hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream) {
     const unsigned gy = (unsigned)((a.bc + BN - 1) / BN);
     // Tile 256 pixels per workgroup only when that still leaves at least two workgroups per CU.
-    const int64_t wg256 = ((a.M + 255) / 256) * gy;
+    const int64_t wg256 = (((int64_t)a.M + 255) / 256) * gy;
     if (wg256 >= 512) {
-        const int64_t gx = (a.M + 255) / 256;
+        const int64_t gx = ((int64_t)a.M + 255) / 256;
         if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
         hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
     } else {
-        const int64_t gx = (a.M + 127) / 128;
+        const int64_t gx = ((int64_t)a.M + 127) / 128;
         hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
     }
     return hipGetLastError();
@@ -255,7 +254,13 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.bw = box.bw;
     a.bh = box.bh;
     a.bc = box.bc;
-    a.M = (int64_t)t.out.n * box.bh * box.bw;
+    const int64_t m64 = (int64_t)t.out.n * box.bh * box.bw;
+    if (m64 >= 0x7fffffffLL) return hipErrorInvalidValue;
+    a.M = (int32_t)m64;
+    a.div_bw = make_fastdiv((uint32_t)box.bw);
+    a.div_bh = make_fastdiv((uint32_t)box.bh);
+    a.div_pitch = make_fastdiv(1);
+    a.div_rows_full = make_fastdiv(1);
     a.KY = t.ky;
     a.KX = t.kx;
     a.SY = t.sy;

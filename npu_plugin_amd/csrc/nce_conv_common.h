@@ -8,6 +8,30 @@ namespace nce {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
+// Division of a 31-bit value by a run-time constant as multiply-high + shift (host-prepared):
+// m = ceil(2^(31+s) / d) with s = ceil(log2 d); q = umulhi(n, m) >> (s - 1). Exact for n < 2^31.
+struct FastDiv {
+    uint32_t d, m, sh;  // m == 0: d == 1
+};
+
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    f.m = 0;
+    f.sh = 0;
+    if (d > 1) {
+        uint32_t s = 0;
+        while ((1ull << s) < d) ++s;
+        f.m = (uint32_t)(((1ull << (31 + s)) + d - 1) / d);
+        f.sh = s - 1;
+    }
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f) {
+    return f.m == 0 ? n : (__umulhi(n, f.m) >> f.sh);
+}
+
 struct ConvArgs {
     const uint8_t* in;
     int64_t in_sn, in_sh, in_sw;
@@ -19,7 +43,8 @@ struct ConvArgs {
     uint8_t* out;
     int64_t out_sn, out_sh, out_sw;
     int32_t x0, y0, z0, bw, bh, bc;
-    int64_t M;  // pixels in the box over all batches
+    int32_t M;  // pixels in the box over all batches (< 2^31)
+    FastDiv div_bw, div_bh, div_pitch, div_rows_full;
     int32_t KY, KX, SY, SX, PT, PL;
     int32_t KG;   // 16-byte groups along K: KY*KX*IC/16
     int32_t ICG;  // 16-byte groups per tap: IC/16
@@ -161,7 +186,6 @@ __device__ __forceinline__ void epi_store(const ConvArgs& a, const EpiSmem& s, v
                                           const int32_t (&acorr)[BF], int mode, const PpeF64& pu) {
     if (mode == PPE_MODE_FOLDED) epi_store_mode<AF, BF, PPE_MODE_FOLDED, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
     else if (mode == PPE_MODE_SLOPE) epi_store_mode<AF, BF, PPE_MODE_SLOPE, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
-    else if (mode == PPE_MODE_ANY_F64) epi_store_mode<AF, BF, PPE_MODE_ANY_F64, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
     else epi_store_mode<AF, BF, PPE_MODE_INT, ACORR>(a, s, acc, ocw, noc, half, dst, valid, acorr, pu);
 }
 

@@ -16,6 +16,7 @@
 #include "nce_conv_common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace nce {
 namespace {
@@ -34,8 +35,6 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* sHalo = smem;
     uint8_t* sWt = smem + a.halo_bytes;
-    int64_t* sSlotOff = reinterpret_cast<int64_t*>(sWt + 2 * WBYTES);
-    int32_t* sFirst = reinterpret_cast<int32_t*>(sSlotOff + a.nslots_max);
     __shared__ int32_t sW2[BN], sBias[BN], sWsum[BN], sCorr[BN];
     __shared__ double sM[BN], sBc[BN];
     const EpiSmem es = {sM, sBc, sW2, sBias, sCorr, sWsum};
@@ -51,111 +50,103 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     const int32_t oc0 = a.z0 + blockIdx.y * BN;
     const int32_t noc = min(BN, a.z0 + a.bc - oc0);
 
+    epi_load_table(a, es, tid, NT, BN, oc0, noc);
+
     // ---- tile geometry (uniform) ------------------------------------------------------------
-    const int64_t m0 = (int64_t)blockIdx.x * BM;
-    const int64_t m_end = min(m0 + (int64_t)BM, a.M);
-    const int64_t rr_first = m0 / a.bw;  // box rows are numbered n * bh + by
-    const int64_t rr_last = (m_end - 1) / a.bw;
-    const int rows_out = (int)(rr_last - rr_first + 1);
-    const int64_t n_first = rr_first / a.bh;
-    const int by_first = (int)(rr_first - n_first * a.bh);
+    const int32_t m0 = blockIdx.x * BM;
+    const int32_t m_end = min(m0 + BM, a.M);
+    const int32_t rr_first = fdiv(m0, a.div_bw);  // box rows are numbered n * bh + by
+    const int32_t rr_last = fdiv(m_end - 1, a.div_bw);
+    const int32_t n_first = fdiv(rr_first, a.div_bh);
+    const int by_first = rr_first - n_first * a.bh;
     const int rows0 = (a.bh - 1 - by_first) * a.SY + a.KY;  // slots of the first image if it runs to its end
     const int rows_full = (a.bh - 1) * a.SY + a.KY;        // slots of a whole image
 
-    auto first_slot_of = [&](int64_t rr) {
-        const int64_t n = rr / a.bh;
-        const int by = (int)(rr - n * a.bh);
-        const int seg = (int)(n - n_first);
+    auto first_slot_of = [&](int32_t rr) {
+        const int32_t n = fdiv(rr, a.div_bh);
+        const int by = rr - n * a.bh;
+        const int seg = n - n_first;
         return seg == 0 ? (by - by_first) * a.SY : rows0 + (seg - 1) * rows_full + by * a.SY;
     };
     const int nslots = first_slot_of(rr_last) + a.KY;
     const int total_h = nslots * a.pitchpx * 4;
 
-    epi_load_table(a, es, tid, NT, BN, oc0, noc);
-    for (int r = tid; r < rows_out; r += NT) sFirst[r] = first_slot_of(rr_first + r);
-    for (int s = tid; s < nslots; s += NT) {
-        int seg, iy;
-        if (s < rows0) {
-            seg = 0;
-            iy = (a.y0 + by_first) * a.SY - a.PT + s;
-        } else {
-            const int q = s - rows0;
-            seg = 1 + q / rows_full;
-            iy = a.y0 * a.SY - a.PT + (q - (seg - 1) * rows_full);
-        }
-        const int64_t n = n_first + seg;
-        sSlotOff[s] = (iy >= 0 && iy < a.H) ? n * a.in_sn + (int64_t)iy * a.in_sh : (int64_t)-1;
-    }
-    __syncthreads();
-
     // ---- staging assignment -------------------------------------------------------------------
     const uint8_t* h_src[JMAX];  // nullptr: fill
     int32_t h_dst[JMAX];         // -1: nothing to stage
-    int32_t h_grp[JMAX];
 #pragma unroll
     for (int j = 0; j < JMAX; ++j) {
         const int h = tid + NT * j;
         h_src[j] = nullptr;
         h_dst[j] = -1;
-        h_grp[j] = h & 3;
         if (h < total_h) {
             const int pxl = h >> 2;
-            const int slot = pxl / a.pitchpx;
+            const int slot = fdiv(pxl, a.div_pitch);
             const int ix = pxl - slot * a.pitchpx - a.PL;
-            const int64_t off = sSlotOff[slot];
+            int seg = 0, iy = (a.y0 + by_first) * a.SY - a.PT + slot;
+            if (slot >= rows0) {
+                const int q = slot - rows0;
+                const int sq = fdiv(q, a.div_rows_full);
+                seg = 1 + sq;
+                iy = a.y0 * a.SY - a.PT + (q - sq * rows_full);
+            }
             h_dst[j] = pxl * 64 + (((h & 3) ^ ((pxl >> 2) & 3)) << 4);
-            if (off >= 0 && ix >= 0 && ix < a.W) h_src[j] = a.in + off + (int64_t)ix * a.in_sw + ((h & 3) << 4);
+            if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W)
+                h_src[j] = a.in + (int64_t)(n_first + seg) * a.in_sn + (int64_t)iy * a.in_sh + (int64_t)ix * a.in_sw + ((h & 3) << 4);
         }
     }
     const uint8_t* w_src[WI];  // nullptr: zero (channel beyond the box)
     int32_t w_dst[WI];
-    int32_t w_row[WI];
-    int32_t w_grp[WI];
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
         const int q = tid + NT * i;
         w_src[i] = nullptr;
         w_dst[i] = -1;
-        w_row[i] = 0;
-        w_grp[i] = q & 3;
         if (q < WCH) {
             const int row = q / (KX * 4);
             const int kx = (q - row * (KX * 4)) >> 2;
             const int lrow = (row & ~31) | row_of_chan(row & 31);
-            w_row[i] = row;
             w_dst[i] = (kx * BN + lrow) * 64 + (((q & 3) ^ ((lrow >> 2) & 3)) << 4);
             if (row < noc) w_src[i] = a.w + (int64_t)(oc0 + row) * a.w_soc + (int64_t)kx * a.IC + ((q & 3) << 4);
         }
     }
+    const int grp16 = (tid & 3) << 4;  // both staging lists give a thread the same 16-byte column (NT % 4 == 0)
 
-    uint4 rw[WI], rh[JMAX];
     const uint4 fill4 = make_uint4(a.fill, a.fill, a.fill, a.fill);
-    auto load_weights = [&](int c, int ky) {
+    const int nsteps = a.nchunks * a.KY;
+    // step index -> (64-channel slice, kernel row)
+    auto load_weights = [&](uint4 (&rw)[WI], int step) {
+        const int c = step / a.KY, ky = step - c * a.KY;
         const int64_t koff = (int64_t)ky * KX * a.IC + c * 64;
+        const bool col_ok = c * 64 + grp16 < a.IC;
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (w_src[i] != nullptr && c * 64 + (w_grp[i] << 4) < a.IC) {
+            if (w_src[i] != nullptr && col_ok && step < nsteps) {
                 v = *reinterpret_cast<const uint4*>(w_src[i] + koff);
                 v.x ^= a.w_xor;
                 v.y ^= a.w_xor;
                 v.z ^= a.w_xor;
                 v.w ^= a.w_xor;
-                if (a.da != 0) atomicAdd(&sWsum[w_row[i]], bytesum(v));
             }
             rw[i] = v;
         }
     };
-    auto store_weights = [&](int buf) {
+    auto store_weights = [&](const uint4 (&rw)[WI], int buf) {
 #pragma unroll
         for (int i = 0; i < WI; ++i)
-            if (w_dst[i] >= 0) *reinterpret_cast<uint4*>(sWt + buf * WBYTES + w_dst[i]) = rw[i];
+            if (w_dst[i] >= 0) {
+                *reinterpret_cast<uint4*>(sWt + buf * WBYTES + w_dst[i]) = rw[i];
+                if (a.da != 0) atomicAdd(&sWsum[(tid + NT * i) / (KX * 4)], bytesum(rw[i]));
+            }
     };
+    uint4 rh[JMAX];
     auto load_halo = [&](int c) {
+        const bool col_ok = c * 64 + grp16 < a.IC;
 #pragma unroll
         for (int j = 0; j < JMAX; ++j) {
             uint4 v = fill4;
-            if (h_src[j] != nullptr && c * 64 + (h_grp[j] << 4) < a.IC) {
+            if (h_src[j] != nullptr && col_ok) {
                 v = *reinterpret_cast<const uint4*>(h_src[j] + c * 64);
                 v.x ^= a.a_xor;
                 v.y ^= a.a_xor;
@@ -171,17 +162,24 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
             if (h_dst[j] >= 0) *reinterpret_cast<uint4*>(sHalo + h_dst[j]) = rh[j];
     };
 
+    // Everything the first step needs is requested before anything is waited for.
+    uint4 rw[WI];
+    load_weights(rw, 0);
+    load_halo(0);
+
     // ---- MFMA operand addressing --------------------------------------------------------------
-    int32_t b_px[BF];      // LDS pixel index of tap (0, 0) for this lane's pixel of fragment x
-    int64_t b_p[BF];       // linear output pixel
+    int32_t b_px[BF];  // LDS pixel index of tap (0, 0) for this lane's pixel of fragment x
+    int32_t b_rr[BF];  // box row and column of that pixel
+    int32_t b_bx[BF];
+    bool valid[BF];
 #pragma unroll
     for (int x = 0; x < BF; ++x) {
-        const int64_t p = m0 + (wp * BF + x) * 32 + l32;
-        b_p[x] = p;
-        const int64_t pc = p < m_end ? p : m_end - 1;  // lanes past the end compute a duplicate
-        const int64_t rr = pc / a.bw;
-        const int bx = (int)(pc - rr * a.bw);
-        b_px[x] = sFirst[(int)(rr - rr_first)] * a.pitchpx + (a.x0 + bx) * a.SX;
+        const int32_t p = m0 + (wp * BF + x) * 32 + l32;
+        valid[x] = p < m_end;
+        const int32_t pc = valid[x] ? p : m_end - 1;  // lanes past the end compute a duplicate
+        b_rr[x] = fdiv(pc, a.div_bw);
+        b_bx[x] = pc - b_rr[x] * a.bw;
+        b_px[x] = first_slot_of(b_rr[x]) * a.pitchpx + (a.x0 + b_bx[x]) * a.SX;
     }
     int32_t a_row[AF];
 #pragma unroll
@@ -195,24 +193,19 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[f][x][v] = 0;
 
-    // ---- main loop: one step = one kernel row (KX taps) of one 64-channel slice --------------
-    const int nsteps = a.nchunks * a.KY;
-    load_weights(0, 0);
-    load_halo(0);
-    store_weights(0);
+    store_weights(rw, 0);
     store_halo();
     __syncthreads();
+
+    // ---- main loop: one step = one kernel row (KX taps) of one 64-channel slice ----------------
+    // The weights of the next step and (on the last kernel row) the halo of the next slice are
+    // requested before this step's MFMAs and written to LDS after them.
     int c = 0, ky = 0;
     for (int s = 0; s < nsteps; ++s) {
-        int c2 = c, ky2 = ky + 1;
-        if (ky2 == a.KY) {
-            ky2 = 0;
-            ++c2;
-        }
-        const bool more = s + 1 < nsteps;
-        const bool new_halo = more && ky2 == 0;
-        if (more) load_weights(c2, ky2);
-        if (new_halo) load_halo(c2);
+        const bool last_row = ky == a.KY - 1;
+        const bool new_halo = last_row && c + 1 < a.nchunks;
+        load_weights(rw, s + 1);
+        if (new_halo) load_halo(c + 1);
 
         const uint8_t* wt = sWt + (s & 1) * WBYTES;
 #pragma unroll
@@ -236,31 +229,30 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
                         acc[f][x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[f], fb[x], acc[f][x], 0, 0, 0);
             }
         }
-        if (more) store_weights((s + 1) & 1);
+        if (s + 1 < nsteps) store_weights(rw, (s + 1) & 1);
         if (new_halo) {
             __syncthreads();  // every wave is done with the current slice
             store_halo();
         }
         __syncthreads();
-        c = c2;
-        ky = ky2;
+        if (last_row) {
+            ky = 0;
+            ++c;
+        } else {
+            ++ky;
+        }
     }
 
     // ---- PPE + store --------------------------------------------------------------------------
     PpeF64 pu;
     const int mode = epi_constants(a, es, tid, NT, BN, &pu);
     uint8_t* dst[BF];
-    bool valid[BF];
     int32_t acorr[BF];
 #pragma unroll
     for (int x = 0; x < BF; ++x) {
-        valid[x] = b_p[x] < m_end;
-        const int64_t pc = valid[x] ? b_p[x] : m_end - 1;
-        const int64_t rr = pc / a.bw;
-        const int bx = (int)(pc - rr * a.bw);
-        const int64_t n = rr / a.bh;
-        const int by = (int)(rr - n * a.bh);
-        dst[x] = a.out + n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+        const int32_t n = fdiv(b_rr[x], a.div_bh);
+        const int by = b_rr[x] - n * a.bh;
+        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + b_bx[x]) * a.out_sw + oc0;
         acorr[x] = 0;
     }
     epi_store<AF, BF, false>(a, es, acc, wn * AF * 32, noc, half, dst, valid, acorr, mode, pu);
@@ -270,10 +262,10 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
 // tile of bm pixels touches (same arithmetic as the kernel).
 void tile_bounds(const ConvArgs& a, int bm, int* rows_max, int* nslots_max) {
     int rmax = 0, smax = 0;
-    const int64_t ntiles = (a.M + bm - 1) / bm;
+    const int64_t ntiles = ((int64_t)a.M + bm - 1) / bm;
     const int rows_full = (a.bh - 1) * a.SY + a.KY;
     for (int64_t t = 0; t < ntiles; ++t) {
-        const int64_t m0 = t * bm, m_end = std::min<int64_t>(m0 + bm, a.M);
+        const int64_t m0 = t * bm, m_end = std::min<int64_t>(m0 + bm, (int64_t)a.M);
         const int64_t rr_first = m0 / a.bw, rr_last = (m_end - 1) / a.bw;
         const int64_t n_first = rr_first / a.bh, n_last = rr_last / a.bh;
         const int by_first = (int)(rr_first - n_first * a.bh), by_last = (int)(rr_last - n_last * a.bh);
@@ -297,10 +289,10 @@ hipError_t try_launch(ConvArgs a, hipStream_t stream, bool* fits) {
     *fits = halo_px * 4 <= (int64_t)JMAX * NT;
     if (!*fits) return hipSuccess;
     a.halo_bytes = (int32_t)(halo_px * 64);
-    const size_t lds = (size_t)a.halo_bytes + 2 * (size_t)BN * KX * 64 + 8 * (size_t)a.nslots_max + 4 * (size_t)a.rows_max + 16;
+    const size_t lds = (size_t)a.halo_bytes + 2 * (size_t)BN * KX * 64;
     *fits = lds <= 140 * 1024;
     if (!*fits) return hipSuccess;
-    const int64_t gx = (a.M + BM - 1) / BM;
+    const int64_t gx = ((int64_t)a.M + BM - 1) / BM;
     const unsigned gy = (unsigned)((a.bc + BN - 1) / BN);
     if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
     auto kernel = &conv_halo_kernel<WN, WP, AF, BF, KX>;
@@ -313,28 +305,40 @@ hipError_t try_launch(ConvArgs a, hipStream_t stream, bool* fits) {
     return hipGetLastError();
 }
 
+// Tile shapes: {channel waves, pixel waves, channel fragments, pixel fragments per wave}.
+//   0: 128 ch x 256 px, 4 waves   1: 64 ch x 256 px, 4 waves   2: 64 ch x 128 px, 4 waves   3: 64 ch x 64 px, 2 waves
+template <int KX>
+hipError_t launch_tile(int tile, const ConvArgs& a, hipStream_t stream, bool* fits) {
+    switch (tile) {
+    case 0: return try_launch<2, 2, 2, 4, KX>(a, stream, fits);
+    case 1: return try_launch<1, 4, 2, 2, KX>(a, stream, fits);
+    case 2: return try_launch<1, 4, 2, 1, KX>(a, stream, fits);
+    default: return try_launch<1, 2, 2, 1, KX>(a, stream, fits);
+    }
+}
+
 template <int KX>
 hipError_t launch_kx(const ConvArgs& a, hipStream_t stream) {
-    // Largest tile that still gives every CU a few workgroups; smaller tiles for small problems.
-    const int64_t wg_big = ((a.M + 255) / 256) * ((a.bc + 127) / 128);
-    const int64_t wg_mid = ((a.M + 255) / 256) * ((a.bc + 63) / 64);
-    const int64_t wg_small = ((a.M + 127) / 128) * ((a.bc + 63) / 64);
-    bool fits = false;
-    hipError_t e;
-    if (a.bc >= 128 && wg_big >= 512) {
-        e = try_launch<2, 2, 2, 4, KX>(a, stream, &fits);
+    // Big tiles pay off only with a long reduction (their epilogue and staging run at one wave per
+    // SIMD); short reductions and small problems take small tiles for occupancy and CU coverage.
+    const int64_t px256 = (a.M + 255) / 256, px128 = (a.M + 127) / 128;
+    const int64_t ch128 = (a.bc + 127) / 128, ch64 = (a.bc + 63) / 64;
+    // Measured on MI355X: 64 ch x 128 px is the best all-round shape; 1x1 kernels with enough
+    // workgroups prefer 64 ch x 256 px. The 128-channel tile (one wave per SIMD) never wins.
+    int first = 2;
+    if (KX == 1 && px256 * ch64 >= 384) first = 1;
+    (void)px128;
+    (void)ch128;
+    static const int forced = [] {
+        const char* e = getenv("NCE_HIP_CONV_TILE");  // tuning knob: force one tile shape (0..3)
+        return e ? atoi(e) : -1;
+    }();
+    if (forced >= 0 && forced <= 3) first = forced;
+    for (int tile = first; tile <= 3; ++tile) {
+        bool fits = false;
+        const hipError_t e = launch_tile<KX>(tile, a, stream, &fits);
         if (fits || e != hipSuccess) return e;
     }
-    if (wg_mid >= 512) {
-        e = try_launch<1, 4, 2, 2, KX>(a, stream, &fits);
-        if (fits || e != hipSuccess) return e;
-    }
-    if (wg_small >= 256) {
-        e = try_launch<1, 4, 2, 1, KX>(a, stream, &fits);
-        if (fits || e != hipSuccess) return e;
-    }
-    e = try_launch<1, 2, 2, 1, KX>(a, stream, &fits);
-    if (fits || e != hipSuccess) return e;
     return hipErrorNotSupported;
 }
 
@@ -344,6 +348,8 @@ hipError_t launch_conv_halo(const ConvArgs& a_in, hipStream_t stream) {
     if (a_in.dw != 0 || a_in.IC < 64) return hipErrorNotSupported;
     ConvArgs a = a_in;
     a.nchunks = (a.IC + 63) / 64;
+    a.div_pitch = make_fastdiv((uint32_t)a.pitchpx);
+    a.div_rows_full = make_fastdiv((uint32_t)((a.bh - 1) * a.SY + a.KY));
     if (a.KX == 1) return launch_kx<1>(a, stream);
     if (a.KX == 3) return launch_kx<3>(a, stream);
     return hipErrorNotSupported;

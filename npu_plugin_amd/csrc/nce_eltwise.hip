@@ -98,7 +98,6 @@ template <bool FLAT>
 void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
     if (path == PPE_MODE_FOLDED) launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
     else if (path == PPE_MODE_SLOPE) launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
-    else if (path == PPE_MODE_ANY_F64) launch_signed<FLAT, PPE_MODE_ANY_F64>(a, grid, s);
     else if (path == PPE_MODE_INT) launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
     else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
@@ -120,16 +119,14 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     a.B = (t.ppe.round_mode == NCE_ROUND_HALF_UP && shift > 0) ? 0.5 : 0.0;
     a.may_sat = shift < kNoSatShift;
     // the same selection the table-driven kernels make per workgroup, made here on the host
-    const bool even = t.ppe.round_mode == NCE_ROUND_HALF_EVEN;
+    const bool half_up = t.ppe.round_mode == NCE_ROUND_HALF_UP;
     const bool prelu = !(t.ppe.prelu_mult == 1 && t.ppe.prelu_shift == 0);
     const int64_t am = t.ppe.prelu_mult < 0 ? -(int64_t)t.ppe.prelu_mult : (int64_t)t.ppe.prelu_mult;
     const bool prelu_sat = am > ((int64_t)1 << t.ppe.prelu_shift);
     int path;
     if (t.table != nullptr) path = PATH_TABLE;
-    else if (shift > kMaxF64Shift) path = PPE_MODE_INT;
-    else if (!even && !a.may_sat && !prelu) path = PPE_MODE_FOLDED;
-    else if (!even && !a.may_sat && prelu && !prelu_sat) path = PPE_MODE_SLOPE;
-    else path = PPE_MODE_ANY_F64;
+    else if (shift > kMaxF64Shift || !half_up || a.may_sat || (prelu && prelu_sat)) path = PPE_MODE_INT;
+    else path = prelu ? PPE_MODE_SLOPE : PPE_MODE_FOLDED;
     if (path == PPE_MODE_FOLDED) a.B += (double)t.ppe.zp_out;
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;

@@ -70,7 +70,9 @@ __device__ __forceinline__ double ppe_scale_B(int32_t bias, double M, int32_t sh
 struct PpeF64 {
     double pm, pc;   // PReLU slope as prelu_mult * 2^-prelu_shift and its rounding constant
     int32_t lo, hi, zp;
+    int32_t lo_zp, hi_zp;  // clamp bounds with the zero point added (folded mode)
     bool even;       // ties-to-even (rint) instead of floor
+    bool round_none; // plain floor
     bool sat;        // requantized value may leave int32: clamp it (some shift < kNoSatShift)
     bool prelu;      // slope differs from identity
     bool prelu_sat;  // slope result may leave int32
@@ -83,12 +85,22 @@ __device__ __forceinline__ PpeF64 ppe_f64_setup(const PpeDev& p, bool may_satura
     u.lo = p.lo;
     u.hi = p.hi;
     u.zp = p.zp_out;
+    u.lo_zp = p.lo + p.zp_out;
+    u.hi_zp = p.hi + p.zp_out;
     u.even = p.round_mode == NCE_ROUND_HALF_EVEN;
+    u.round_none = p.round_mode == NCE_ROUND_NONE;
     u.sat = may_saturate;
     u.prelu = !(p.prelu_mult == 1 && p.prelu_shift == 0);
     const int64_t am = p.prelu_mult < 0 ? -(int64_t)p.prelu_mult : (int64_t)p.prelu_mult;
     u.prelu_sat = am > ((int64_t)1 << p.prelu_shift);
     return u;
+}
+
+// clamp(y, lo, hi) for lo <= hi in one instruction
+__device__ __forceinline__ int32_t med3_i32(int32_t y, int32_t lo, int32_t hi) {
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(y), "v"(lo), "v"(hi));
+    return r;
 }
 
 __device__ __forceinline__ double clamp_i32_range(double v) {
@@ -108,45 +120,32 @@ __device__ __forceinline__ int32_t ppe_finish_f64_t(double v, const PpeF64& u) {
         if (PSAT) r = clamp_i32_range(r);
         v = v < 0.0 ? r : v;
     }
-    int32_t y = (int32_t)v;  // in range by construction
-    y = y < u.lo ? u.lo : (y > u.hi ? u.hi : y);
-    return y + u.zp;
+    const int32_t y = (int32_t)v;  // in range by construction
+    return med3_i32(y, u.lo, u.hi) + u.zp;
 }
 
 // Fastest form: round half-up, no saturation, no slope, and the output zero point already folded into
 // B and into the clamp bounds (floor(x + zp) = floor(x) + zp for an integer zp).
 __device__ __forceinline__ int32_t ppe_finish_f64_folded(double v, int32_t lo_zp, int32_t hi_zp) {
-    const int32_t y = (int32_t)__builtin_floor(v);
-    return y < lo_zp ? lo_zp : (y > hi_zp ? hi_zp : y);
+    return med3_i32((int32_t)__builtin_floor(v), lo_zp, hi_zp);
 }
 
-// Which specialisation a workgroup runs (uniform). 0: folded fast path, 1: half-up + slope,
-// 2: any flags (run-time selects), 3: integer arithmetic.
-enum { PPE_MODE_FOLDED = 0, PPE_MODE_SLOPE = 1, PPE_MODE_ANY_F64 = 2, PPE_MODE_INT = 3 };
+// Which specialisation a workgroup runs (uniform). FOLDED and SLOPE cover rounding half-up without
+// int32 saturation (every shift >= 18), with or without a negative slope; every other combination
+// (ties-to-even, floor, tiny shifts, slopes that can overflow) runs the integer path.
+enum { PPE_MODE_FOLDED = 0, PPE_MODE_SLOPE = 1, PPE_MODE_INT = 3 };
 
 __device__ __forceinline__ int ppe_mode_of(const PpeF64& u, bool use_int) {
-    if (use_int) return PPE_MODE_INT;
-    if (!u.even && !u.sat && !u.prelu) return PPE_MODE_FOLDED;
-    if (!u.even && !u.sat && u.prelu && !u.prelu_sat) return PPE_MODE_SLOPE;
-    return PPE_MODE_ANY_F64;
+    if (use_int || u.even || u.sat || u.round_none) return PPE_MODE_INT;
+    if (!u.prelu) return PPE_MODE_FOLDED;
+    if (!u.prelu_sat) return PPE_MODE_SLOPE;
+    return PPE_MODE_INT;
 }
 
 template <int MODE>
 __device__ __forceinline__ int32_t ppe_finish_mode(double v, const PpeF64& u) {
-    if (MODE == PPE_MODE_FOLDED) return ppe_finish_f64_folded(v, u.lo + u.zp, u.hi + u.zp);
-    if (MODE == PPE_MODE_SLOPE) return ppe_finish_f64_t<false, false, true, false>(v, u);
-    // run-time flags
-    v = u.even ? __builtin_rint(v) : __builtin_floor(v);
-    if (u.sat) v = clamp_i32_range(v);
-    if (u.prelu) {
-        double r = __builtin_fma(v, u.pm, u.pc);
-        r = u.even ? __builtin_rint(r) : __builtin_floor(r);
-        if (u.prelu_sat) r = clamp_i32_range(r);
-        v = v < 0.0 ? r : v;
-    }
-    int32_t y = (int32_t)v;
-    y = y < u.lo ? u.lo : (y > u.hi ? u.hi : y);
-    return y + u.zp;
+    if (MODE == PPE_MODE_FOLDED) return ppe_finish_f64_folded(v, u.lo_zp, u.hi_zp);
+    return ppe_finish_f64_t<false, false, true, false>(v, u);
 }
 
 // B constant of a channel for the given mode: the folded mode carries the output zero point.

@@ -218,7 +218,6 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         const int chl = cg << 4;
         if (pmode == PPE_MODE_FOLDED) requant16<PPE_MODE_FOLDED>(acc, sM + chl, sB + chl, pu, wo);
         else if (pmode == PPE_MODE_SLOPE) requant16<PPE_MODE_SLOPE>(acc, sM + chl, sB + chl, pu, wo);
-        else if (pmode == PPE_MODE_ANY_F64) requant16<PPE_MODE_ANY_F64>(acc, sM + chl, sB + chl, pu, wo);
         else {
             wo[0] = wo[1] = wo[2] = wo[3] = 0;
 #pragma unroll
