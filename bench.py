@@ -145,17 +145,26 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-others", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-reference", action="store_true",
+                    help="also run plain 256 MiB device copies, the known-size reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported (no collectives, no sharding).")
 
-    import torch  # noqa: F401  (device memory and streams)
+    import torch  # device memory and streams
 
     import npu_plugin_amd as nce
     workloads = make_workloads()
     if args.workload not in workloads:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(workloads)}")
     ex = nce.Executor(device_id=0, log_level=1)
+    if args.traffic_reference:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(7)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     maker, bound = workloads[args.workload]
     case, main_res = measure(ex, args.workload, maker, bound, args.steps, args.warmup)

@@ -48,6 +48,19 @@ struct TaskDev {
     PpeDev ppe;
 };
 
+// MI355X spreads consecutive workgroup ids over its 8 XCDs (id % 8), each with a private L2. Tiles that
+// share input rows should share an L2, so kernels walk their tiles in this order: XCD x gets the
+// contiguous range [x * per_xcd, (x + 1) * per_xcd). Launch 8 * per_xcd workgroups, per_xcd =
+// ceil(ntiles / 8); ids mapped at or beyond ntiles have nothing to do.
+constexpr int kNumXcd = 8;
+__host__ __device__ inline uint32_t xcd_grid(uint32_t ntiles) {
+    return kNumXcd * ((ntiles + kNumXcd - 1) / kNumXcd);
+}
+__device__ inline uint32_t xcd_tile(uint32_t block_id, uint32_t ntiles) {
+    const uint32_t per_xcd = (ntiles + kNumXcd - 1) / kNumXcd;
+    return (block_id % kNumXcd) * per_xcd + block_id / kNumXcd;
+}
+
 hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);
 hipError_t launch_pool(const TaskDev& t, const Box& box, bool is_max, hipStream_t stream);
 hipError_t launch_dwconv(const TaskDev& t, const Box& box, hipStream_t stream);

@@ -41,7 +41,10 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
     const int half = lane >> 5;
     const int l32 = lane & 31;
 
-    const int32_t m0 = blockIdx.x * BM;
+    const uint32_t ntiles = ((uint32_t)a.M + BM - 1) / BM;
+    const uint32_t tile = xcd_tile(blockIdx.x, ntiles);
+    if (tile >= ntiles) return;  // uniform for the whole workgroup
+    const int32_t m0 = tile * BM;
     const int32_t oc0 = a.z0 + blockIdx.y * BN;
     const int32_t noc = min(BN, a.z0 + a.bc - oc0);
 
@@ -223,10 +226,10 @@ hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream) {
     if (wg256 >= 512) {
         const int64_t gx = ((int64_t)a.M + 255) / 256;
         if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
     } else {
         const int64_t gx = ((int64_t)a.M + 127) / 128;
-        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3((unsigned)gx, gy), dim3(NTHREADS), 0, stream, a);
+        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
     }
     return hipGetLastError();
 }

@@ -50,10 +50,14 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     const int32_t oc0 = a.z0 + blockIdx.y * BN;
     const int32_t noc = min(BN, a.z0 + a.bc - oc0);
 
+    const uint32_t ntiles = ((uint32_t)a.M + BM - 1) / BM;
+    const uint32_t tile = xcd_tile(blockIdx.x, ntiles);
+    if (tile >= ntiles) return;  // uniform for the whole workgroup
+
     epi_load_table(a, es, tid, NT, BN, oc0, noc);
 
     // ---- tile geometry (uniform) ------------------------------------------------------------
-    const int32_t m0 = blockIdx.x * BM;
+    const int32_t m0 = tile * BM;
     const int32_t m_end = min(m0 + BM, a.M);
     const int32_t rr_first = fdiv(m0, a.div_bw);  // box rows are numbered n * bh + by
     const int32_t rr_last = fdiv(m_end - 1, a.div_bw);
@@ -301,7 +305,7 @@ hipError_t try_launch(ConvArgs a, hipStream_t stream, bool* fits) {
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)gx, gy), dim3(NT), lds, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((unsigned)gx), gy), dim3(NT), lds, stream, a);
     return hipGetLastError();
 }
 

@@ -61,6 +61,7 @@ struct WinArgs {
     Box box;
     int64_t npix;
     int32_t items_per_thread;
+    uint32_t nblocks;  // item blocks per channel slab (the grid is padded to a multiple of the XCD count)
     uint32_t a_xor;   // 0x80808080 for i8 activations
     uint32_t fill;    // word of re-biased zero-point bytes for out-of-image taps
     int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     __syncthreads();
 
     const int64_t nitems = a.npix * nslab;
-    const int64_t first = (int64_t)blockIdx.x * NT * a.items_per_thread;
+    const int64_t first = (int64_t)xcd_tile(blockIdx.x, a.nblocks) * NT * a.items_per_thread;
     for (int it = 0; it < a.items_per_thread; ++it) {
         const int64_t item = first + (int64_t)it * NT + threadIdx.x;
         if (item >= nitems) break;
@@ -243,7 +244,8 @@ hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
     const int64_t items = a.npix * (cgroups < SLAB_GROUPS ? cgroups : SLAB_GROUPS);
     a.items_per_thread = items > (int64_t)NT * 8192 ? 4 : 1;
     const int64_t blocks = (items + NT * a.items_per_thread - 1) / (NT * a.items_per_thread);
-    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (blocks > 0x7ffffff0LL) return hipErrorInvalidValue;
+    a.nblocks = (uint32_t)blocks;
     a.a_xor = t.in.is_signed ? 0x80808080u : 0u;
     a.zpu = t.in.zp + (t.in.is_signed ? 128 : 0);
     a.fill = (uint32_t)a.zpu * 0x01010101u;
@@ -253,7 +255,7 @@ hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((window_kernel<MODE>), dim3((unsigned)blocks, (unsigned)nslabs), dim3(NT), lds, s, a);
+    hipLaunchKernelGGL((window_kernel<MODE>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
     return hipGetLastError();
 }
 
