@@ -115,7 +115,9 @@ __device__ __forceinline__ int epi_constants(const ConvArgs& a, const EpiSmem& s
         const int32_t w2 = s.w2[c];
         const int32_t shift = table_shift(w2);
         bad_shift |= shift > kMaxF64Shift;
-        small_shift |= shift < kNoSatShift;
+        // |acc| <= K * 255 * 255 (and never beyond int32: the accumulator wraps)
+        const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
+        small_shift |= ppe_may_saturate(acc_bound, s.bias[c], table_mult(w2), shift);
     }
     const bool use_int = __syncthreads_or(bad_shift) != 0;
     const bool may_sat = __syncthreads_or(small_shift) != 0;

@@ -117,7 +117,7 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     const int shift = t.ppe.quant_shift;
     a.M = ldexp((double)t.ppe.quant_mult, -shift);
     a.B = (t.ppe.round_mode == NCE_ROUND_HALF_UP && shift > 0) ? 0.5 : 0.0;
-    a.may_sat = shift < kNoSatShift;
+    a.may_sat = ppe_may_saturate(((int64_t)t.ppe.in1_mult + t.ppe.in2_mult) * 255, 0, t.ppe.quant_mult, shift);
     // the same selection the table-driven kernels make per workgroup, made here on the host
     const bool half_up = t.ppe.round_mode == NCE_ROUND_HALF_UP;
     const bool prelu = !(t.ppe.prelu_mult == 1 && t.ppe.prelu_shift == 0);

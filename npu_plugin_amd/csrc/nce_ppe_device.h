@@ -20,7 +20,13 @@
 namespace nce {
 
 constexpr int kMaxF64Shift = 52;  // largest shift for which the FP64 formulation is exact
-constexpr int kNoSatShift = 18;   // |x * mult| < 2^48, so >> 18 or more cannot leave int32
+
+// Can round_shift((acc + bias) * mult, shift) leave int32 for any |acc| <= acc_bound ?
+// (It cannot once shift >= 18, because |x * mult| < 2^48; smaller shifts are fine for small sums.)
+__host__ __device__ inline bool ppe_may_saturate(int64_t acc_bound, int32_t bias, int32_t mult, int32_t shift) {
+    const int64_t b = acc_bound + (bias < 0 ? -(int64_t)bias : (int64_t)bias);
+    return ((b * (int64_t)mult) >> shift) + 1 >= 2147483647LL;
+}
 
 __device__ __forceinline__ int64_t rshift_round(int64_t p, int32_t s, int32_t mode) {
     if (s <= 0) return p;
@@ -73,7 +79,7 @@ struct PpeF64 {
     int32_t lo_zp, hi_zp;  // clamp bounds with the zero point added (folded mode)
     bool even;       // ties-to-even (rint) instead of floor
     bool round_none; // plain floor
-    bool sat;        // requantized value may leave int32: clamp it (some shift < kNoSatShift)
+    bool sat;        // the requantized value may leave int32 (see ppe_may_saturate)
     bool prelu;      // slope differs from identity
     bool prelu_sat;  // slope result may leave int32
 };
@@ -96,11 +102,10 @@ __device__ __forceinline__ PpeF64 ppe_f64_setup(const PpeDev& p, bool may_satura
     return u;
 }
 
-// clamp(y, lo, hi) for lo <= hi in one instruction
+// clamp(y, lo, hi) for lo <= hi. Plain min/max (not inline asm) so that the scheduler stays free to
+// interleave the independent per-element chains.
 __device__ __forceinline__ int32_t med3_i32(int32_t y, int32_t lo, int32_t hi) {
-    int32_t r;
-    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(y), "v"(lo), "v"(hi));
-    return r;
+    return min(max(y, lo), hi);
 }
 
 __device__ __forceinline__ double clamp_i32_range(double v) {

@@ -87,10 +87,15 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     int bad_shift = 0, small_shift = 0;
     if (MODE != MODE_MAX) {
         for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
-            int32_t shift = t.ppe.quant_shift;
-            if (t.table != nullptr) shift = table_shift(t.table[(int64_t)(box.z0 + slab0 * 16 + ch) * t.table_stride + 2]);
+            int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
+            if (t.table != nullptr) {
+                const int32_t* row = t.table + (int64_t)(box.z0 + slab0 * 16 + ch) * t.table_stride;
+                mult = table_mult(row[2]);
+                shift = table_shift(row[2]);
+                bias = row[3];
+            }
             bad_shift |= shift > kMaxF64Shift;
-            small_shift |= shift < kNoSatShift;
+            small_shift |= ppe_may_saturate((int64_t)ntaps * (MODE == MODE_DW ? 65025 : 255), bias, mult, shift);
         }
     }
     const bool use_int = __syncthreads_or(bad_shift) != 0;
