@@ -23,7 +23,15 @@ PEAK_HBM_GBS = 8000.0    # MI355X HBM3E, GB/s
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); filled
 # per workload once measured, None otherwise.
-MEASURED_TRAFFIC = {}
+# Scale factors from the 256 MiB copy in the same runs: FETCH_SIZE reads 131085 KiB for 262144 KiB
+# fetched (x2.0), WRITE_SIZE reads 262144 KiB (x1.0). Values in bytes per launch.
+MEASURED_TRAFFIC = {
+    "cfg2": int((1094.1 * 2.0 + 1568.0) * 1024),
+    "cfg3_dw": int((9496.6 * 2.0 + 4704.0) * 1024),
+    "cfg3_maxpool": int((2413.4 * 2.0 + 1176.0) * 1024),
+    "cfg3_avgpool": int((660.3 * 2.0 + 294.0) * 1024),
+    "cfg4": int((3158.6 * 2.0 + 3136.0) * 1024),
+}
 
 
 def make_workloads():
@@ -83,7 +91,34 @@ def measure(ex, name, maker, bound, steps, warmup):
                   "bytes_per_step": nbytes, "roofline": roof}
 
 
-def measure_graph(ex, steps, warmup, batch=32):
+def per_layer_table(ex, dg, reps=10):
+    """HIP-event time of every task of the graph, run alone `reps` times back to back."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    g = dg.graph
+    rows = []
+    for L, task in zip(g.layers, dg.tasks):
+        tl = ex.task_list()
+        for _ in range(reps):
+            tl.append(task)
+        tl.enqueue(stream)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        tl.enqueue(stream)
+        e1.record()
+        torch.cuda.synchronize()
+        tl.destroy()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        n, oh, ow, oc = g.tensors[L.dst]
+        ops = 2 * n * oh * ow * oc * L.kernel[0] * L.kernel[1] * L.real_ic if L.task_type == 0 else 0
+        rows.append({"layer": L.name, "task_type": L.task_type, "out": [n, oh, ow, oc], "kernel": L.kernel,
+                     "strides": L.strides, "in_ch": g.tensors[L.src][3], "us": us, "tops": ops / us / 1e6,
+                     "gbs": g.layer_bytes(L) / us / 1e3})
+    return rows
+
+
+def measure_graph(ex, steps, warmup, batch=32, per_layer=False):
     """cfg5: the whole ResNet-50 task graph (53 convs + max pool + 16 adds) as one step."""
     import torch
     from npu_plugin_amd import workloads as W
@@ -108,8 +143,13 @@ def measure_graph(ex, steps, warmup, batch=32):
     roof = {"bound": "mfma", "achieved": ops / ev / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
             "frac": ops / ev / 1e12 / PEAK_INT8_TOPS, "traffic": None, "kernel_us": ev * 1e6,
             "note": "whole graph per step: 53 conv kernels + 1 max pool + 16 adds, launched back to back"}
+    layers = per_layer_table(ex, dg) if per_layer else None
+    if layers:
+        for r in layers:
+            print(f"{r['layer']:22s} type {r['task_type']} in_ch {r['in_ch']:5d} out {r['out']} k {r['kernel']} s {r['strides']} "
+                  f"{r['us']:8.1f} us {r['tops']:7.1f} TOP/s {r['gbs']:7.0f} GB/s", file=sys.stderr)
     dg.task_list.destroy()
-    return {"workload": f"cfg5_resnet50_b{batch}_224 (70 tasks)", "value": ops / wall / 1e9, "unit": "GOPS",
+    return {"workload": f"cfg5_resnet50_b{batch}_224 (70 tasks)", "steps": steps, "value": ops / wall / 1e9, "unit": "GOPS",
             "ms_per_step": wall * 1e3, "ops_per_step": ops, "conv_bytes_per_step": conv_bytes,
             "pool_add_bytes_per_step": other_bytes, "roofline": roof}
 
@@ -145,6 +185,7 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-others", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--per-layer", action="store_true", help="cfg5: print a per-task timing table on stderr")
     ap.add_argument("--traffic-reference", action="store_true",
                     help="also run plain 256 MiB device copies, the known-size reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -155,8 +196,8 @@ def main():
 
     import npu_plugin_amd as nce
     workloads = make_workloads()
-    if args.workload not in workloads:
-        sys.exit(f"unknown workload {args.workload}; choose from {sorted(workloads)}")
+    if args.workload not in workloads and args.workload != "cfg5":
+        sys.exit(f"unknown workload {args.workload}; choose from {sorted(workloads) + ['cfg5']}")
     ex = nce.Executor(device_id=0, log_level=1)
     if args.traffic_reference:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(7)
@@ -166,14 +207,21 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    maker, bound = workloads[args.workload]
-    case, main_res = measure(ex, args.workload, maker, bound, args.steps, args.warmup)
+    if args.workload == "cfg5":
+        case, bound = None, "mfma"
+        main_res = measure_graph(ex, max(5, args.steps // 10), max(2, args.warmup // 10), per_layer=args.per_layer)
+        main_res["bytes_per_step"] = main_res["conv_bytes_per_step"] + main_res["pool_add_bytes_per_step"]
+        workload_name = main_res["workload"]
+    else:
+        maker, bound = workloads[args.workload]
+        case, main_res = measure(ex, args.workload, maker, bound, args.steps, args.warmup)
+        workload_name = case.name
     line = {
         "metric": "INT8 GOPS & % MFMA peak (conv); GB/s & % HBM peak (dw/pool/eltwise)",
         "value": main_res["value"],
         "unit": main_res["unit"],
         "n_gpus": 1,
-        "steps": args.steps,
+        "steps": main_res.get("steps", args.steps),
         "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": True,
@@ -181,10 +229,10 @@ def main():
         "vs_baseline": None,
         "dtype": "int8 (u8 x i8 -> i32 accumulate, integer PPE)",
         "data": "synthetic (seeded uniform u8 activations, i8 weights, random per-channel mult/shift tables)",
-        "config": {"workload": case.name, "ops_per_step": main_res["ops_per_step"], "bytes_per_step": main_res["bytes_per_step"]},
+        "config": {"workload": workload_name, "ops_per_step": main_res["ops_per_step"], "bytes_per_step": main_res["bytes_per_step"]},
         "roofline": main_res["roofline"],
     }
-    if not args.no_cpu:
+    if not args.no_cpu and case is not None:
         line["cpu_baseline"] = cpu_baseline(case, bound)
     if not args.no_others:
         others = {}
@@ -193,7 +241,8 @@ def main():
                 continue
             _, r = measure(ex, name, mk, bd, args.steps, args.warmup)
             others[name] = r
-        others["cfg5"] = measure_graph(ex, max(5, args.steps // 10), max(2, args.warmup // 10))
+        if args.workload != "cfg5":
+            others["cfg5"] = measure_graph(ex, max(5, args.steps // 10), max(2, args.warmup // 10))
         line["other_workloads"] = others
     ex.destroy()
     print(json.dumps(line))
