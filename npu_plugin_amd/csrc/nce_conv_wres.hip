@@ -1,0 +1,488 @@
+// CONV task, weights-resident implicit GEMM on v_mfma_i32_16x16x64_i8.
+//
+// A workgroup owns one slice of 16*NF output channels and a run of pixel tiles. It stages the WHOLE
+// reduction (KY*KX*IC bytes) of its channels in LDS once, already in MFMA operand order, and after that
+// single barrier its wavefronts never synchronise again: each wave walks its own tiles of 16*BF output
+// pixels, loads the activation operand straight from global memory in the layout the matrix
+// instruction wants, and runs the fused PPE on its accumulators.
+//
+// Why 16x16x64: the B operand of that instruction is 16 pixels x 64 reduction bytes with lane
+// (c = lane % 16, q = lane / 16) holding bytes 16q..16q+15 of pixel c. For NHWC activations those are
+// the four 16-byte quarters of one pixel's 64 consecutive channels, so the 64 lanes of one load cover
+// whole 64-byte runs (a contiguous KiB when IC == 64) instead of 32 half-used lines, and the result
+// layout (lane holds rows 4q..4q+3 of column c) lets the four lanes of a pixel store 64 consecutive
+// output bytes.
+//
+// The reduction is cut in steps of 64 bytes = four 16-byte units; unit u covers bytes 16u..16u+15 of
+// the OYXI weight row, i.e. tap u / (IC/16), input channels 16 * (u % (IC/16)). With IC a multiple of
+// 64 a step never straddles taps and the tap bookkeeping is scalar; other channel counts take the
+// per-lane path (template MODE 2). Semantics and the fused PPE are the ones of nce_conv.hip.
+#include "nce_conv_common.h"
+
+#include <algorithm>
+#include <cstdlib>
+
+namespace nce {
+namespace {
+
+struct WresArgs {
+    ConvArgs a;
+    int32_t k16;        // 16-byte units along the reduction
+    int32_t nsteps;     // 64-byte steps (k16 rounded up to 4), padded to a multiple of the load depth
+    int32_t ntaps;      // KY * KX
+    int32_t nc64;       // 64-byte chunks along IC (fast path)
+    uint32_t ntiles;    // pixel tiles of 16*BF pixels
+    uint32_t ngroups;   // workgroups along pixels
+    int32_t tpg;        // tiles per workgroup
+    int32_t lu;         // log2 of the units one wave-load covers per weight row
+    int32_t lnblk;      // log2 of the row blocks of a channel slice (64 >> lu rows each)
+    int32_t ui;         // unit passes per row: ceil(nsteps * 4 / 2^lu)
+    FastDiv div_icg;    // by IC / 16
+    FastDiv div_kx;     // by KX
+};
+
+enum { WRES_FAST = 0, WRES_FAST_MASK = 1, WRES_GENERIC = 2 };
+
+// One 64-byte line per byte value: lanes whose tap lies outside the image load the input zero point from
+// here instead of the activation tensor, so every activation load is unconditional (nothing has to
+// wait for it until the matrix instruction that consumes it).
+struct FillTable {
+    uint8_t b[256][64];
+};
+constexpr FillTable make_fill_table() {
+    FillTable t{};
+    for (int v = 0; v < 256; ++v)
+        for (int i = 0; i < 64; ++i) t.b[v][i] = (uint8_t)v;
+    return t;
+}
+__device__ const FillTable g_fill = make_fill_table();
+
+// Channel (within the slice) that row i of channel fragment f carries: lane (c, q) of the result then
+// holds channels 4*NF*q .. 4*NF*q + 4*NF-1, consecutive, for f = 0..NF-1 and its 4 registers.
+template <int NF>
+__device__ __forceinline__ void frag_of_channel(int ch, int* f, int* i) {
+    const int qp = ch / (4 * NF);
+    const int rem = ch - qp * (4 * NF);
+    *f = rem >> 2;
+    *i = 4 * qp + (rem & 3);
+}
+
+// bits [lo, hi) of a 32-bit mask (empty when hi <= lo; hi - lo <= 32)
+__device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
+    return hi > lo ? ((0xFFFFFFFFu >> (32 - (hi - lo))) << lo) : 0u;
+}
+
+template <int NF, int BF, int PMODE>
+__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBz, const double* sMd,
+                                              const v4i (&acc)[NF][BF], const v4i (&wsum)[NF], int q, int noc,
+                                              uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu) {
+    const int ch0 = 4 * NF * q;
+    if (ch0 >= noc) return;
+    uint32_t wo[BF][NF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+        // The constants are re-read from LDS for every tile: hoisted out of the tile loop they would
+        // occupy up to 96 registers for the whole kernel.
+        __asm__ volatile("" ::: "memory");
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = ch0 + 4 * f + r;
+            double M = 0.0, B = 0.0;
+            int32_t w2 = 0, bias = 0, corr = 0;
+            // the activation zero point enters as da * (sum of the channel's weights)
+            if (PMODE == PPE_MODE_INT) {
+                w2 = s.w2[c];
+                bias = s.bias[c];
+                corr = a.da * wsum[f][r];  // |da| <= 255, |sum w'| < 2^23
+            } else {
+                M = s.M[c];
+                B = PMODE == PPE_MODE_FOLDED ? sBz[c] : s.B[c];  // the folded mode carries the output zero point in B
+                B = __builtin_fma((double)wsum[f][r], sMd[c], B);  // exact: 24 x 25 significant bits
+            }
+#pragma unroll
+            for (int x = 0; x < BF; ++x) {
+                const int32_t av = acc[f][x][r];
+                int32_t y;
+                if (PMODE == PPE_MODE_INT)
+                    y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
+                else
+                    y = ppe_finish_mode<PMODE>(__builtin_fma((double)av, M, B), pu);
+                const uint32_t b = (uint32_t)y & 0xFFu;
+                wo[x][f] = r == 0 ? b : (wo[x][f] | (b << (8 * r)));
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // one fragment's constants live at a time
+    }
+#pragma unroll
+    for (int x = 0; x < BF; ++x) {
+        if (!valid[x]) continue;
+        if constexpr (NF == 4) *reinterpret_cast<uint4*>(dst[x] + ch0) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
+        else *reinterpret_cast<uint2*>(dst[x] + ch0) = make_uint2(wo[x][0], wo[x][1]);
+    }
+}
+
+// D: reduction steps whose activation loads are in flight per wave; the host pads the step count to a
+// multiple of D (the padding steps multiply zero weights by the fill line).
+template <int NF, int BF, int MODE, int D>
+__global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
+    constexpr int OCT = 16 * NF;
+    constexpr int BP = 16 * BF;
+    constexpr int WB = 8;      // weight loads in flight per lane while staging
+    static_assert(NF == 2 || NF == 4, "channel fragments");
+    const ConvArgs& a = w.a;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
+    __shared__ int32_t sW2[OCT], sBias[OCT];
+    __shared__ double sM[OCT], sBc[OCT], sBz[OCT], sMd[OCT];  // scale, bias term, same plus zero point, scale * da
+    __shared__ int32_t sFlags;
+    const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps the tile walk in scalar registers
+    const int nwaves = blockDim.x >> 6;
+    const int c16 = lane & 15;
+    const int q = lane >> 4;
+
+    const int32_t oc0 = a.z0 + blockIdx.y * OCT;
+    const int32_t noc = min(OCT, a.z0 + a.bc - oc0);
+    const uint32_t group = xcd_tile(blockIdx.x, w.ngroups);
+    if (group >= w.ngroups) return;  // uniform for the whole workgroup
+
+    const int axor = (int)a.a_xor;
+    const uint8_t* const fillp = &g_fill.b[(a.fill ^ a.a_xor) & 0xFFu][q * 16];
+    const int S = w.nsteps;
+    const uint32_t t_end = min((group + 1) * (uint32_t)w.tpg, w.ntiles);
+    uint32_t t = group * (uint32_t)w.tpg + wave;
+
+    // state of the tile in flight
+    const uint8_t* pbase[BF];
+    uint8_t* dst[BF];
+    bool valid[BF];
+    uint32_t mask0[BF], mask1[BF];  // FAST_MASK: tap bits; GENERIC: row bits, column bits
+    int32_t it_ky = 0, it_kx = 0, it_c64 = 0, it_tap = 0, ls = 0;  // (tap, chunk) the next load belongs to
+    int64_t it_off = 0;
+    v4i fb[D][BF];
+
+    auto setup = [&]() {
+#pragma unroll
+        for (int x = 0; x < BF; ++x) {
+            const int32_t p = (int32_t)t * BP + 16 * x + c16;
+            valid[x] = p < a.M;
+            const int32_t pc = valid[x] ? p : a.M - 1;  // lanes past the end compute a duplicate
+            const int32_t rr = fdiv(pc, a.div_bw);
+            const int32_t bx = pc - rr * a.bw;
+            const int32_t n = fdiv(rr, a.div_bh);
+            const int32_t by = rr - n * a.bh;
+            const int32_t iy0 = (a.y0 + by) * a.SY - a.PT;
+            const int32_t ix0 = (a.x0 + bx) * a.SX - a.PL;
+            pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + (MODE == WRES_GENERIC ? 0 : q * 16);
+            dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+            mask0[x] = mask1[x] = 0;
+            if (MODE != WRES_FAST) {
+                const uint32_t rows = bit_range(max(0, -iy0), min(a.KY, a.H - iy0));
+                const uint32_t cols = bit_range(max(0, -ix0), min(a.KX, a.W - ix0));
+                if (MODE == WRES_GENERIC) {
+                    mask0[x] = rows;
+                    mask1[x] = cols;
+                } else {
+                    uint32_t m = 0;
+                    for (int ky = a.KY - 1; ky >= 0; --ky) m = (m << a.KX) | (((rows >> ky) & 1u) ? cols : 0u);
+                    mask0[x] = m;
+                }
+            }
+        }
+        it_ky = it_kx = it_c64 = it_tap = ls = 0;
+        it_off = 0;
+    };
+    // Request the activation operand of the next step for every pixel fragment (raw bytes).
+    auto load_b = [&](v4i (&d)[BF]) {
+        if (MODE == WRES_GENERIC) {
+            const int u = 4 * ls + q;
+            const int tap = fdiv(u, w.div_icg);
+            const int icg = u - tap * a.ICG;
+            const int ky = fdiv(tap, w.div_kx);
+            const int kx = tap - ky * a.KX;
+            const int64_t off = (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + icg * 16;
+#pragma unroll
+            for (int x = 0; x < BF; ++x) {
+                const bool ok = u < w.k16 && ((mask0[x] >> ky) & (mask1[x] >> kx) & 1u) != 0;
+                const uint8_t* src = ok ? pbase[x] + off : fillp;
+                d[x] = *reinterpret_cast<const v4i*>(src);
+            }
+            ++ls;
+        } else {
+#pragma unroll
+            for (int x = 0; x < BF; ++x) {
+                // (a padding step re-reads tap 0, whose weights it multiplies are zero; with masks its bit is clear)
+                const uint8_t* src = pbase[x] + it_off;
+                if (MODE == WRES_FAST_MASK) src = ((mask0[x] >> it_tap) & 1u) ? src : fillp;
+                d[x] = *reinterpret_cast<const v4i*>(src);
+            }
+            it_off += 64;
+            if (++it_c64 == w.nc64) {
+                it_c64 = 0;
+                ++it_tap;
+                if (++it_kx == a.KX) {
+                    it_kx = 0;
+                    ++it_ky;
+                }
+                it_off = (int64_t)it_ky * a.in_sh + (int64_t)it_kx * a.in_sw;
+                if (it_tap >= w.ntaps) {  // padding steps: stay on a readable address
+                    it_off = 0;
+                    it_tap = 31;
+                }
+            }
+        }
+    };
+    auto first_loads = [&]() {
+#pragma unroll
+        for (int j = 0; j < D; ++j) load_b(fb[j]);
+    };
+    // The first tile's activations are requested before anything is waited for.
+    if (t < t_end) {
+        setup();
+        first_loads();
+    }
+
+    // ---- stage the channel slice's weights in operand order; per-channel constants ---------------
+    // Lanes split into 64/U rows x U consecutive 16-byte units (U = 2^w.lu covers a row, or is 64), so the
+    // loads of a row are contiguous. A (pass, row block) pair is one such wave-wide load; the first lane
+    // of a row in the last pass also derives the row's PPE constants from its weight-table entry.
+    {
+        const int lu = w.lu;
+        const int U = 1 << lu;
+        const int sub = lane & (U - 1);
+        const int rsub = lane >> lu;
+        const int lnblk = w.lnblk;
+        const int k16p = S * 4;
+        const int npairs = w.ui << lnblk;
+        const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
+        // The last wave also derives the per-channel PPE constants (lane = channel) while its weight
+        // loads are in flight.
+        const bool consts_wave = wave == nwaves - 1;
+        int32_t tw2 = 0, tbias = 0;
+        if (consts_wave && lane < noc) {
+            const int32_t* trow = a.table + (int64_t)(oc0 + lane) * a.table_stride;
+            tw2 = trow[2];
+            tbias = trow[3];
+        }
+        auto do_consts = [&]() {
+            const int32_t mult = table_mult(tw2), shift = table_shift(tw2);
+            const bool bad = lane < OCT && shift > kMaxF64Shift;
+            const bool sat = lane < OCT && ppe_may_saturate(acc_bound, tbias, mult, shift);
+            const int wf = (__any(bad) ? 1 : 0) | (__any(sat) ? 2 : 0);
+            if (lane == 0) sFlags = wf;
+            if (lane < OCT) {
+                const double M = ppe_scale_M(mult, shift);
+                const double B = ppe_scale_B(tbias, M, shift, a.ppe.round_mode);
+                sW2[lane] = tw2;
+                sBias[lane] = tbias;
+                sM[lane] = M;
+                sMd[lane] = M * (double)a.da;
+                sBc[lane] = B;
+                sBz[lane] = B + (double)a.ppe.zp_out;
+            }
+        };
+        for (int m0 = wave; m0 < npairs; m0 += nwaves * WB) {
+            // requests only (nothing here consumes a loaded value) ...
+            uint4 v[WB];
+#pragma unroll
+            for (int j = 0; j < WB; ++j) {
+                const int m = m0 + j * nwaves;
+                const int row = ((m & ((1 << lnblk) - 1)) << (6 - lu)) + rsub;
+                const int u = ((m >> lnblk) << lu) + sub;
+                v[j] = make_uint4(0, 0, 0, 0);
+                if (m < npairs && row < noc && u < w.k16)
+                    v[j] = *reinterpret_cast<const uint4*>(a.w + (int64_t)(oc0 + row) * a.w_soc + (int64_t)u * 16);
+            }
+            if (consts_wave && m0 == wave) do_consts();
+            // ... then the LDS writes
+#pragma unroll
+            for (int j = 0; j < WB; ++j) {
+                const int m = m0 + j * nwaves;
+                const int row = ((m & ((1 << lnblk) - 1)) << (6 - lu)) + rsub;
+                const int u = ((m >> lnblk) << lu) + sub;
+                if (m < npairs && u < k16p) {
+                    int f, i;
+                    frag_of_channel<NF>(row, &f, &i);
+                    uint4 x = v[j];
+                    if (row < noc && u < w.k16) {
+                        x.x ^= a.w_xor;
+                        x.y ^= a.w_xor;
+                        x.z ^= a.w_xor;
+                        x.w ^= a.w_xor;
+                    }
+                    *reinterpret_cast<uint4*>(sWt + (((u >> 2) * NF + f) * 64 + (u & 3) * 16 + i) * 16) = x;
+                }
+            }
+        }
+        if (consts_wave && wave >= npairs) do_consts();  // this wave had no weights to stage
+    }
+    __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
+
+    const int flags = sFlags;
+    const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
+    const int pmode = ppe_mode_of(pu, (flags & 1) != 0);
+
+    // ---- per-wave tile loop -----------------------------------------------------------------------
+    // The per-channel weight sums come out of the matrix unit as well: in its first tile a wave also
+    // multiplies every weight fragment by an all-ones operand (each column of the result is the sum).
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    v4i wsum[NF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) wsum[f] = v4i{0, 0, 0, 0};
+    bool sum_pass = a.da != 0;
+    while (t < t_end) {
+        v4i acc[NF][BF];
+#pragma unroll
+        for (int f = 0; f < NF; ++f)
+#pragma unroll
+            for (int x = 0; x < BF; ++x) acc[f][x] = v4i{0, 0, 0, 0};
+        // Steady state: every step consumes one ring slot and refills it for step + D, with no branch
+        // around the load, so that the wait before a step covers exactly the loads older than its own.
+        const uint8_t* ap = sWt + lane * 16;
+        v4i fa[NF];
+#pragma unroll
+        for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
+        auto step = [&](v4i (&b)[BF], bool more_a) {
+#pragma unroll
+            for (int x = 0; x < BF; ++x) b[x] = b[x] ^ axor;
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+#pragma unroll
+                for (int x = 0; x < BF; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], b[x], acc[f][x], 0, 0, 0);
+            if (sum_pass) {
+#pragma unroll
+                for (int f = 0; f < NF; ++f) wsum[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], ones, wsum[f], 0, 0, 0);
+            }
+            ap += NF * 1024;
+            if (more_a) {
+#pragma unroll
+                for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
+            }
+        };
+        for (int g = D; g < S; g += D) {
+#pragma unroll
+            for (int j = 0; j < D; ++j) {
+                step(fb[j], true);
+                load_b(fb[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < D; ++j) step(fb[j], j + 1 < D);
+        sum_pass = false;
+        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
+        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
+        t += nwaves;
+        if (t < t_end) {
+            setup();
+            first_loads();
+        }
+    }
+}
+
+constexpr size_t kWresLdsCap = 148 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
+
+template <int NF, int BF, int MODE, int D>
+hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t stream) {
+    constexpr int OCT = 16 * NF;
+    constexpr int BP = 16 * BF;
+    const ConvArgs& a = w.a;
+    w.ntiles = (uint32_t)(((int64_t)a.M + BP - 1) / BP);
+    w.tpg = nwaves * tiles_per_wave;
+    w.ngroups = (w.ntiles + w.tpg - 1) / w.tpg;
+    const unsigned gy = (unsigned)((a.bc + OCT - 1) / OCT);
+    w.nsteps = (w.nsteps + D - 1) / D * D;
+    const size_t lds = (size_t)w.nsteps * NF * 1024;
+    if (lds > kWresLdsCap) return hipErrorNotSupported;
+    const int k16p = w.nsteps * 4;
+    w.lu = 2;
+    while (w.lu < 6 && (1 << w.lu) < k16p) ++w.lu;
+    w.lnblk = (NF == 4 ? 6 : 5) - 6 + w.lu;
+    w.ui = (k16p + (1 << w.lu) - 1) >> w.lu;
+    auto kernel = &conv_wres_kernel<NF, BF, MODE, D>;
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
+    return hipGetLastError();
+}
+
+template <int NF, int BF>
+hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
+    // Load depth: 4 steps when that needs no padding step (and the ring fits the registers), else 2.
+    constexpr int DMAX = BF == 4 ? 2 : 4;
+    if (DMAX == 4 && w.nsteps % 4 == 0) {
+        if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, DMAX>(w, nwaves, tpw, stream);
+        if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, DMAX>(w, nwaves, tpw, stream);
+        return launch_one<NF, BF, WRES_GENERIC, DMAX>(w, nwaves, tpw, stream);
+    }
+    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, 2>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, 2>(w, nwaves, tpw, stream);
+    return launch_one<NF, BF, WRES_GENERIC, 2>(w, nwaves, tpw, stream);
+}
+
+template <int NF>
+hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream) {
+    if (bf == 4) return launch_mode<NF, 4>(w, mode, nwaves, tpw, stream);
+    if (bf == 2) return launch_mode<NF, 2>(w, mode, nwaves, tpw, stream);
+    return launch_mode<NF, 1>(w, mode, nwaves, tpw, stream);
+}
+
+}  // namespace
+
+hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
+    if (a.dw != 0 || a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
+    WresArgs w;
+    w.a = a;
+    w.k16 = a.KG;
+    w.nsteps = (a.KG + 3) / 4;
+    w.nc64 = a.IC / 64;
+    w.ntaps = a.KY * a.KX;
+    w.div_icg = make_fastdiv((uint32_t)a.ICG);
+    w.div_kx = make_fastdiv((uint32_t)a.KX);
+    const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
+    if (wl2 > kWresLdsCap) return hipErrorNotSupported;
+
+    // every tap of every output pixel of the box inside the image?
+    const int64_t iy_lo = (int64_t)a.y0 * a.SY - a.PT, iy_hi = (int64_t)(a.y0 + a.bh - 1) * a.SY - a.PT + a.KY - 1;
+    const int64_t ix_lo = (int64_t)a.x0 * a.SX - a.PL, ix_hi = (int64_t)(a.x0 + a.bw - 1) * a.SX - a.PL + a.KX - 1;
+    const bool inside = iy_lo >= 0 && iy_hi < a.H && ix_lo >= 0 && ix_hi < a.W;
+    const int mode = (a.IC % 64 != 0) ? WRES_GENERIC : (inside ? WRES_FAST : WRES_FAST_MASK);
+    if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return hipErrorNotSupported;  // one bit per tap, bit 31 stays clear
+
+    // Shape of the work: nf channel fragments per slice, bf pixel fragments per wave tile. Measured on
+    // MI355X over the ResNet-50 layer shapes, the best shape is always the LARGEST tile that still
+    // yields about 1500 wave tiles (six waves per CU, one round of workgroups); beyond that, waves take
+    // several tiles each rather than the grid growing.
+    auto wave_tiles = [&](int nf, int bf) {
+        return (((int64_t)a.M + 16 * bf - 1) / (16 * bf)) * ((a.bc + 16 * nf - 1) / (16 * nf));
+    };
+    const bool nf4_ok = wl4 <= kWresLdsCap && a.bc > 32;
+    const int64_t want = 1500;
+    int nf = nf4_ok ? 4 : 2, bf = 4;
+    while (bf > 1 && wave_tiles(nf, bf) < want) bf >>= 1;
+    if (nf == 4 && wave_tiles(nf, bf) < want) nf = 2;
+    const int nwaves = 8;
+    int tpw = (int)std::max<int64_t>(1, wave_tiles(nf, bf) / 1568);
+
+    int nw = nwaves;
+    static const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning knob: "nf,bf,nwaves,tiles_per_wave"
+    if (forced) {
+        int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
+        if (sscanf(forced, "%d,%d,%d,%d", &fnf, &fbf, &fnw, &ftpw) == 4) {
+            if ((fnf == 2 || (fnf == 4 && wl4 <= kWresLdsCap))) nf = fnf;
+            if (fbf == 1 || fbf == 2 || fbf == 4) bf = fbf;
+            if (fnw >= 1 && fnw <= 8) nw = fnw;
+            if (ftpw >= 1) tpw = ftpw;
+        }
+    }
+    if (nf == 4) return launch_bf<4>(w, bf, mode, nw, tpw, stream);
+    return launch_bf<2>(w, bf, mode, nw, tpw, stream);
+}
+
+}  // namespace nce
