@@ -285,10 +285,9 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.nslots_max = a.rows_max = a.nchunks = a.halo_bytes = 0;
     a.ppe = t.ppe;
     if (a.M == 0 || box.bc == 0) return hipSuccess;
-    static const int path = [] {
-        const char* e = getenv("NCE_HIP_CONV_PATH");  // tuning knob: 1 = skip the weights-resident kernel, 2 = gather only
-        return e ? atoi(e) : 0;
-    }();
+    // tuning and test knob: 1 = skip the weights-resident kernel, 2 = gather kernel only
+    const char* path_env = getenv("NCE_HIP_CONV_PATH");
+    const int path = path_env ? atoi(path_env) : 0;
     hipError_t e = path == 0 ? launch_conv_wres(a, stream) : hipErrorNotSupported;
     if (e != hipErrorNotSupported) return e;
     e = path <= 1 ? launch_conv_halo(a, stream) : hipErrorNotSupported;

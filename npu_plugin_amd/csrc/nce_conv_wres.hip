@@ -471,7 +471,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     int tpw = (int)std::max<int64_t>(1, wave_tiles(nf, bf) / 1568);
 
     int nw = nwaves;
-    static const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning knob: "nf,bf,nwaves,tiles_per_wave"
+    const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning and test knob: "nf,bf,nwaves,tiles_per_wave"
     if (forced) {
         int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
         if (sscanf(forced, "%d,%d,%d,%d", &fnf, &fbf, &fnw, &ftpw) == 4) {

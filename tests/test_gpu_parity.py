@@ -254,7 +254,59 @@ def test_resnet50_graph_every_tensor(executor, batch, size):
     dg.task_list.destroy()
 
 
+# ---- weights-resident conv kernel: every instantiation (channel fragments x pixel fragments x path) ---
+
+WRES_CONFIGS = ["4,4,8,1", "4,2,8,2", "4,1,4,1", "2,4,8,1", "2,2,4,3", "2,1,8,1"]  # nf, bf, waves, tiles per wave
+WRES_SHAPES = [
+    # (n, h, w, ic, oc, k, s, pads, in_zp)
+    (2, 20, 20, 64, 64, (1, 1), (1, 1), (0, 0, 0, 0), 128),    # one reduction step (padded to two), no masks
+    (2, 20, 20, 256, 80, (1, 1), (1, 1), (0, 0, 0, 0), 5),     # four steps (deep ring), weight sums, ragged channels
+    (3, 19, 17, 64, 48, (3, 3), (1, 1), (1, 1, 1, 1), 128),    # tap masks, odd step count, partial pixel tile
+    (2, 21, 21, 128, 64, (3, 3), (2, 2), (1, 1, 1, 1), 200),   # stride 2 with masks and weight sums
+    (2, 30, 30, 16, 64, (7, 7), (2, 2), (3, 3, 3, 3), 114),    # per-lane tap path: 16 channels, 49 taps
+    (2, 12, 12, 48, 32, (3, 3), (1, 1), (1, 1, 1, 1), 77),     # per-lane tap path: steps straddle taps
+    (1, 9, 9, 64, 16, (3, 3), (1, 1), (0, 0, 0, 0), 128),      # 3x3 without padding: every tap inside
+    (2, 10, 10, 192, 144, (1, 1), (2, 2), (0, 0, 0, 0), 0),    # 1x1 stride 2, three steps padded to four
+]
+
+
+@pytest.mark.parametrize("config", WRES_CONFIGS)
+@pytest.mark.parametrize("shape", WRES_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
+def test_conv_weights_resident_instantiations(executor, monkeypatch, shape, config):
+    n, h, w, ic, oc, k, s, pads, in_zp = shape
+    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    check(K.conv_case(400 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=in_zp, out_zp=9,
+                      ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
+
+
+@pytest.mark.parametrize("config", ["4,2,8,1", "2,1,4,2"])
+def test_conv_weights_resident_types_and_modes(executor, monkeypatch, config):
+    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    check(K.conv_case(421, 2, 14, 14, 64, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128), executor)
+    check(K.conv_case(422, 2, 14, 14, 64, 64, w_signed=False, w_zp=128, in_zp=121), executor)
+    check(K.conv_case(423, 2, 14, 14, 64, 64, in_zp=3, ppe=dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255,
+                                                                 round_mode=nce.ROUND_HALF_EVEN)), executor)   # integer PPE path
+    check(K.conv_case(424, 2, 14, 14, 64, 64, in_zp=3, scale_lo=20.0, scale_hi=255.0), executor)               # may saturate int32
+    check(K.conv_case(425, 2, 14, 14, 64, 64, in_zp=250, ppe=dict(mode=nce.PPE_NOOP, clamp_low=128, clamp_high=255)), executor)
+
+
+def test_conv_weights_resident_variants(executor, monkeypatch):
+    monkeypatch.setenv("NCE_HIP_CONV_WRES", "2,2,4,1")
+    test_conv_halo_variants(executor)
+
+
 # ---- halo-staged conv kernel: every tile configuration, image-crossing tiles, partial slices -----
+# (the dispatcher prefers the weights-resident kernel; NCE_HIP_CONV_PATH=1 sends these to the halo kernel)
+
+@pytest.fixture
+def halo_path(monkeypatch):
+    monkeypatch.setenv("NCE_HIP_CONV_PATH", "1")
+
+
+@pytest.fixture
+def gather_path(monkeypatch):
+    monkeypatch.setenv("NCE_HIP_CONV_PATH", "2")
+
 
 HALO_CASES = [
     # (n, h, w, ic, oc, k, s, pads)                      which tile the dispatcher picks
@@ -277,13 +329,13 @@ HALO_CASES = [
 
 
 @pytest.mark.parametrize("shape", HALO_CASES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}s{s[6][0]}")
-def test_conv_halo_kernel_shapes(executor, shape):
+def test_conv_halo_kernel_shapes(executor, halo_path, shape):
     n, h, w, ic, oc, k, s, pads = shape
     check(K.conv_case(200 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14)), executor)
 
 
-def test_conv_halo_zero_points_and_types(executor):
+def test_conv_halo_zero_points_and_types(executor, halo_path):
     check(K.conv_case(301, 2, 20, 20, 64, 64, in_zp=3, out_zp=17), executor)                      # weight-sum correction
     check(K.conv_case(302, 2, 20, 20, 128, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128), executor)
     check(K.conv_case(303, 2, 20, 20, 64, 64, w_signed=False, w_zp=128, in_zp=121), executor)
@@ -301,3 +353,20 @@ def test_conv_halo_variants(executor):
     from oracle import nce_oracle
     nce_oracle.run(K.build_task(part, part.input, part.weights, part.table, canvas))
     assert np.array_equal(K.run_hip(part, executor), canvas)
+
+
+def test_conv_halo_variants_on_halo_path(executor, halo_path):
+    test_conv_halo_variants(executor)
+
+
+@pytest.mark.parametrize("shape", [HALO_CASES[3], HALO_CASES[6], HALO_CASES[10], HALO_CASES[12]],
+                         ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}s{s[6][0]}")
+def test_conv_gather_kernel_shapes(executor, gather_path, shape):
+    n, h, w, ic, oc, k, s, pads = shape
+    check(K.conv_case(500 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=77,
+                      ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14)), executor)
+
+
+def test_conv_wide_kernel_falls_back(executor):
+    # 7x7 with 64 input channels needs more than 31 tap bits: the halo / gather kernels take it
+    check(K.conv_case(511, 1, 20, 20, 64, 32, k=(7, 7), s=(1, 1), pads=(3, 3, 3, 3), in_zp=100), executor)
