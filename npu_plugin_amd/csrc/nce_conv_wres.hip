@@ -72,18 +72,39 @@ __device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
     return hi > lo ? ((0xFFFFFFFFu >> (32 - (hi - lo))) << lo) : 0u;
 }
 
+// Wave-uniform constants of the packed FP epilogue: after floor() the value goes to FP32 (exact below
+// 2^24, monotone beyond, and everything beyond is clamped anyway), is clamped with one v_med3_f32 into
+// 0..255 and lands in its output byte with v_cvt_pk_u8_f32. Signed outputs are computed 128 higher
+// and flipped back by an XOR on the packed word.
+struct EpiPack {
+    float lo, hi, zp;   // clamp bounds and zero point, including the +128 of signed outputs
+    uint32_t flip;      // 0x80808080 for signed outputs
+    double zp_fold;     // folded mode: what B carries on top of the bias term
+};
+
+__device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
+    EpiPack e;
+    const int32_t sb = pu.lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
+    e.lo = (float)(pu.lo_zp + sb);
+    e.hi = (float)(pu.hi_zp + sb);
+    e.zp = (float)(pu.zp + sb);
+    e.flip = sb ? 0x80808080u : 0u;
+    e.zp_fold = (double)(pu.zp + sb);
+    return e;
+}
+
 template <int NF, int BF, int PMODE>
-__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBz, const double* sMd,
+__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sMd,
                                               const v4i (&acc)[NF][BF], const v4i (&wsum)[NF], int q, int noc,
-                                              uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu) {
+                                              uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
+                                              const EpiPack& ep) {
     const int ch0 = 4 * NF * q;
     if (ch0 >= noc) return;
     uint32_t wo[BF][NF];
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-        // The constants are re-read from LDS for every tile: hoisted out of the tile loop they would
-        // occupy up to 96 registers for the whole kernel.
-        __asm__ volatile("" ::: "memory");
+#pragma unroll
+        for (int x = 0; x < BF; ++x) wo[x][f] = 0;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int c = ch0 + 4 * f + r;
@@ -96,20 +117,33 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
                 corr = a.da * wsum[f][r];  // |da| <= 255, |sum w'| < 2^23
             } else {
                 M = s.M[c];
-                B = PMODE == PPE_MODE_FOLDED ? sBz[c] : s.B[c];  // the folded mode carries the output zero point in B
-                B = __builtin_fma((double)wsum[f][r], sMd[c], B);  // exact: 24 x 25 significant bits
+                B = __builtin_fma((double)wsum[f][r], sMd[c], s.B[c]);  // exact: 24 x 25 significant bits
+                if (PMODE == PPE_MODE_FOLDED) B += ep.zp_fold;          // floor(x + zp) = floor(x) + zp
             }
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
                 const int32_t av = acc[f][x][r];
-                int32_t y;
-                if (PMODE == PPE_MODE_INT)
-                    y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
-                else
-                    y = ppe_finish_mode<PMODE>(__builtin_fma((double)av, M, B), pu);
-                const uint32_t b = (uint32_t)y & 0xFFu;
-                wo[x][f] = r == 0 ? b : (wo[x][f] | (b << (8 * r)));
+                if (PMODE == PPE_MODE_INT) {
+                    const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
+                    wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
+                } else {
+                    double v = __builtin_floor(__builtin_fma((double)av, M, B));
+                    float y;
+                    if (PMODE == PPE_MODE_SLOPE) {
+                        const double neg = __builtin_floor(__builtin_fma(v, pu.pm, pu.pc));
+                        v = v < 0.0 ? neg : v;
+                        y = (float)v + ep.zp;
+                    } else {
+                        y = (float)v;
+                    }
+                    y = __builtin_amdgcn_fmed3f(y, ep.lo, ep.hi);
+                    wo[x][f] = __builtin_amdgcn_cvt_pk_u8_f32(y, r, wo[x][f]);
+                }
             }
+        }
+        if (PMODE != PPE_MODE_INT) {
+#pragma unroll
+            for (int x = 0; x < BF; ++x) wo[x][f] ^= ep.flip;
         }
         __builtin_amdgcn_sched_barrier(0);  // one fragment's constants live at a time
     }
@@ -133,7 +167,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
     __shared__ int32_t sW2[OCT], sBias[OCT];
-    __shared__ double sM[OCT], sBc[OCT], sBz[OCT], sMd[OCT];  // scale, bias term, same plus zero point, scale * da
+    __shared__ double sM[OCT], sBc[OCT], sMd[OCT];  // scale, bias term, scale * da
     __shared__ int32_t sFlags;
     const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
 
@@ -281,10 +315,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 sM[lane] = M;
                 sMd[lane] = M * (double)a.da;
                 sBc[lane] = B;
-                sBz[lane] = B + (double)a.ppe.zp_out;
             }
         };
-        for (int m0 = wave; m0 < npairs; m0 += nwaves * WB) {
+        // (runs at least once: the constants wave may have no weights to stage)
+        for (int m0 = wave, first = 1; first || m0 < npairs; m0 += nwaves * WB, first = 0) {
             // requests only (nothing here consumes a loaded value) ...
             uint4 v[WB];
 #pragma unroll
@@ -296,7 +330,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 if (m < npairs && row < noc && u < w.k16)
                     v[j] = *reinterpret_cast<const uint4*>(a.w + (int64_t)(oc0 + row) * a.w_soc + (int64_t)u * 16);
             }
-            if (consts_wave && m0 == wave) do_consts();
+            if (first && consts_wave) do_consts();  // between the weight requests and their use
             // ... then the LDS writes
 #pragma unroll
             for (int j = 0; j < WB; ++j) {
@@ -317,13 +351,13 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 }
             }
         }
-        if (consts_wave && wave >= npairs) do_consts();  // this wave had no weights to stage
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
 
     const int flags = sFlags;
     const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
     const int pmode = ppe_mode_of(pu, (flags & 1) != 0);
+    const EpiPack ep = epi_pack_setup(pu);
 
     // ---- per-wave tile loop -----------------------------------------------------------------------
     // The per-channel weight sums come out of the matrix unit as well: in its first tile a wave also
@@ -372,9 +406,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 #pragma unroll
         for (int j = 0; j < D; ++j) step(fb[j], j + 1 < D);
         sum_pass = false;
-        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
-        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
-        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBz, sMd, acc, wsum, q, noc, dst, valid, pu);
+        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
+        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
         t += nwaves;
         if (t < t_end) {
             setup();
