@@ -1,4 +1,4 @@
-"""ctypes view of include/nce_hip.h and include/nce_params.h, and the loader of libnce_hip.so.
+"""ctypes view of include/nce_hip.h, nce_params.h and nce_hwtest.h, and the loader of libnce_hip.so.
 
 The shared library is the product: loading fails loudly when it has not been built, and nothing
 here falls back to a CPU implementation.
@@ -119,6 +119,49 @@ class Quant(C.Structure):
 
 # Every symbol the two headers declare: name -> (restype, argtypes)
 _P = C.POINTER
+class HwtestLayer(C.Structure):
+    _fields_ = [
+        ("present", C.c_int32),
+        ("dtype", C.c_int32),
+        ("dtype_name", C.c_char * 16),
+        ("shape", C.c_int64 * 4),
+        ("has_quant", C.c_int32),
+        ("num_scales", C.c_int32),
+        ("scale0", C.c_double),
+        ("zero_point", C.c_int64),
+        ("low_range", C.c_int64),
+        ("high_range", C.c_int64),
+        ("file_path", C.c_char * 256),
+    ]
+
+
+class HwtestCase(C.Structure):
+    _fields_ = [
+        ("arch", C.c_int32),
+        ("case_type", C.c_char * 48),
+        ("task_type", C.c_int32),
+        ("input", HwtestLayer),
+        ("weight", HwtestLayer),
+        ("output", HwtestLayer),
+        ("kernel", C.c_int32 * 2),
+        ("stride", C.c_int32 * 2),
+        ("pad", C.c_int32 * 4),
+        ("group", C.c_int32),
+        ("dilation", C.c_int32),
+        ("compress", C.c_int32),
+        ("act_sparsity", C.c_int32),
+        ("mpe_mode", C.c_int32),
+        ("activation", C.c_int32),
+        ("alpha", C.c_double),
+        ("maximum", C.c_double),
+        ("output_order", C.c_char * 8),
+        ("ew_mode", C.c_char * 8),
+    ]
+
+
+# nce_hwtest_activation_t
+HWTEST_ACT_NONE, HWTEST_ACT_RELU, HWTEST_ACT_RELUX, HWTEST_ACT_LEAKY_RELU, HWTEST_ACT_OTHER = range(5)
+
 SYMBOLS = {
     "nceGetVersion": (C.c_int, [_P(C.c_uint32), _P(C.c_uint32)]),
     "nceExecutorCreate": (C.c_int, [ExecutorDesc, _P(C.c_void_p), _P(C.c_void_p)]),
@@ -140,6 +183,12 @@ SYMBOLS = {
     "ncePpeForAvgPool": (C.c_int, [C.c_int32, Quant, Quant, C.c_int32, C.c_int32, C.c_int32, C.c_double, C.c_double,
                                    _P(PpeTask)]),
     "ncePpeForEltwiseAdd": (C.c_int, [C.c_int32, Quant, Quant, Quant, C.c_int32, C.c_double, C.c_double, _P(PpeTask)]),
+    "nceHwtestParse": (C.c_int, [C.c_char_p, _P(C.c_void_p), C.c_void_p]),
+    "nceHwtestDestroy": (C.c_int, [C.c_void_p]),
+    "nceHwtestGetCase": (C.c_int, [C.c_void_p, _P(HwtestCase)]),
+    "nceHwtestGetScales": (C.c_int, [C.c_void_p, C.c_int32, _P(C.c_double), C.c_int32]),
+    "nceHwtestBuildTask": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc), _P(DpuTask), _P(PpeTask), _P(C.c_int32), C.c_int32,
+                                     _P(C.c_int32), C.c_void_p]),
 }
 
 _lib = None

@@ -10,25 +10,7 @@
 #include <vector>
 
 #include "nce_common.h"
-
-struct nce_log_s {
-    std::mutex mu;
-    std::string text;
-    int level = 1;
-
-    void add(int lvl, const char* fmt, ...) {
-        if (lvl > level) return;
-        char buf[1024];
-        va_list ap;
-        va_start(ap, fmt);
-        vsnprintf(buf, sizeof(buf), fmt, ap);
-        va_end(ap);
-        std::lock_guard<std::mutex> lk(mu);
-        if (text.size() > (1u << 20)) text.clear();  // bounded
-        text += buf;
-        text += '\n';
-    }
-};
+#include "nce_log.h"
 
 struct nce_executor_s {
     int device = 0;

@@ -1,0 +1,231 @@
+"""The hwtest-JSON front end (include/nce_hwtest.h): parsing with the reference's keys and error messages, and the
+descriptors its builders produce. CPU tests check parsed fields and generated parameters against values the
+reference's own sources fix; the GPU tests run the built tasks and compare with the oracle."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import npu_plugin_amd as nce
+from npu_plugin_amd import _abi as abi
+from npu_plugin_amd import hwtest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hwtest")
+
+
+def load(name):
+    return open(os.path.join(GOLDEN, name)).read()
+
+
+def word2(mult, shift):
+    return np.array([(mult << 16) | (shift << 8)], dtype=np.uint32).view(np.int32)[0]
+
+
+# ---- parser ------------------------------------------------------------------------------------------
+
+def test_reference_parser_unit_test_document():
+    # what the reference's own unit test asserts after parsing this document
+    # (test_case_json_parser_unit_test.cpp:221-226): input dtype "uint8", weight scale {0.01}
+    case = hwtest.parse(load("reference_parser_unit_test.json"))
+    assert case.info.input.dtype_name == b"uint8" and case.info.input.dtype == abi.DT_U8
+    assert case.scales(1) == [0.01]
+    assert case.case_type == "ZMajorConvolution" and case.arch == abi.ARCH_VPUX37XX and case.output_order == "nhwc"
+    assert list(case.info.input.shape) == [1, 256, 16, 16] and list(case.info.weight.shape) == [64, 256, 1, 1]
+    assert case.info.input.zero_point == 127 and (case.info.input.low_range, case.info.input.high_range) == (0, 255)
+    assert list(case.info.stride) == [1, 1] and list(case.info.pad) == [0, 0, 0, 0] and case.info.group == 1
+    # that document writes "output" as an object, which loadOutputLayer (getArray) does not see
+    assert case.info.output.present == 0
+
+
+def test_reference_vpuip_fixture_is_rejected_like_the_reference_does():
+    # the file predates the current schema: no "architecture" -> TestCaseJsonDescriptor::parse throws
+    with pytest.raises(nce.NCEError) as e:
+        hwtest.parse(load("reference_vpuip_conv2d_u8_to_u8.json"))
+    assert e.value.code == abi.ERROR_INVALID_ARGUMENT and "Failed to get architecture" in e.value.log
+
+
+@pytest.mark.parametrize("mutate,message", [
+    (lambda d: d.update(architecture="VPUX99XX"), "Failed to parse architecture"),
+    (lambda d: d.pop("compiler_backend"), "Failed to get compiler_backend"),
+    (lambda d: d.update(compiler_backend="LLVM"), "Failed to parse compiler_backend"),
+    (lambda d: d.pop("case_type"), "Failed to get case type"),
+    (lambda d: d.update(case_type="Conv2DU8"), "Unsupported case type: Conv2DU8"),
+    (lambda d: d.pop("conv_op"), "loadConvLayer: missing conv_op config"),
+    (lambda d: d["conv_op"].pop("stride"), "loadConvLayer: missing strides"),
+    (lambda d: d["conv_op"].pop("pad"), "loadConvLayer: missing pads"),
+    (lambda d: d["input"][0].pop("shape"), "loadInputLayer: missing shape"),
+    (lambda d: d["weight"][0]["quantization"].pop("scale"), "loadQuantizationParams: cannot find scale config param"),
+    (lambda d: d.update(output_order="hwcn"), "ODUPermutation value not supported: hwcn"),
+])
+def test_parse_errors_carry_the_reference_messages(mutate, message):
+    d = json.loads(load("zmajor_conv_u8.json"))
+    mutate(d)
+    with pytest.raises(nce.NCEError) as e:
+        hwtest.parse(json.dumps(d))
+    assert e.value.code == abi.ERROR_INVALID_ARGUMENT and message in e.value.log
+
+
+def test_comment_lines_names_and_other_case_types():
+    text = "// RUN: vpux-translate --import-HWTEST %s\n   // second comment\n" + load("zmajor_conv_u8.json")
+    case = hwtest.parse(text)
+    assert case.task_type == abi.TASK_CONV
+    for bad in ("", "   \n// only a comment\n", "[1, 2]", '{"architecture": "VPUX37XX",}'):
+        with pytest.raises(nce.NCEError):
+            hwtest.parse(bad)
+    d = json.loads(load("zmajor_conv_u8.json"))
+    d.update(case_type="zmajorconvolution", compiler_backend="elf", output_order="NHWC")  # names compare case-insensitively
+    d["activation"] = {"name": "PReLU", "alpha": 0.25, "max": 6}
+    case = hwtest.parse(json.dumps(d))
+    assert case.task_type == abi.TASK_CONV and case.info.activation == abi.HWTEST_ACT_LEAKY_RELU
+    assert case.info.alpha == 0.25 and case.info.maximum == 6.0
+    d = {"architecture": "VPUX37XX", "compiler_backend": "ELF", "case_type": "ActShave"}
+    case = hwtest.parse(json.dumps(d))  # recognised, but not an NCE task
+    assert case.task_type == -1
+    with pytest.raises(nce.NCEError) as e:
+        case.build_task(np.zeros(16, np.uint8), None, np.zeros(16, np.uint8))
+    assert e.value.code == abi.ERROR_UNSUPPORTED
+
+
+# ---- builders ----------------------------------------------------------------------------------------
+
+def buffers(case, rng):
+    i, w, o = case.info.input, case.info.weight, case.info.output
+    n, c, h, wd = i.shape
+    x = rng.integers(0, 256, (n, h, wd, c), dtype=np.uint8)
+    out = np.zeros((o.shape[0], o.shape[2], o.shape[3], o.shape[1]), dtype=np.uint8)
+    wt = None
+    if case.task_type == abi.TASK_CONV:
+        dt = np.int8 if w.dtype == abi.DT_I8 else np.uint8
+        wt = rng.integers(-127 if dt == np.int8 else 0, 128 if dt == np.int8 else 256, (w.shape[0], w.shape[2], w.shape[3], w.shape[1])).astype(dt)
+    elif case.task_type == abi.TASK_DWCONV:
+        taps = int(w.shape[2] * w.shape[3])
+        wt = np.zeros((w.shape[0], 16 * ((taps + 15) // 16)), dtype=np.int8)
+        wt[:, :taps] = rng.integers(-127, 128, (w.shape[0], taps))
+    elif case.task_type == abi.TASK_ELTWISE:
+        wt = rng.integers(0, 256, x.shape, dtype=np.uint8)
+    return x, wt, out
+
+
+def test_zmajor_conv_descriptor_follows_the_builder(validator):
+    case = hwtest.parse(load("zmajor_conv3x3_lrelu_per_channel.json"))
+    x, wt, out = buffers(case, np.random.default_rng(1))
+    task = case.build_task(x, wt, out)
+    d = task.desc
+    assert d.task_type == abi.TASK_CONV and list(d.kernel_size) == [3, 3] and list(d.kernel_strides) == [1, 1]
+    assert (d.kernel_pad_left, d.kernel_pad_right, d.kernel_pad_top, d.kernel_pad_bottom) == (1, 1, 1, 1)
+    assert list(d.weights.dims) == [48, 64, 3, 3] and list(d.weights.strides_bytes) == [576, 1, 192, 64]  # OYXI
+    v = task._variants[0]
+    assert list(v.out_start) == [0, 0, 0] and list(v.out_end) == [17, 17, 47] and v.mpe_mode == abi.MPE_CUBOID_8x16
+    p = task._ppe
+    # storage-domain clamp, LPRELU with PReLUApproximation(0.1) = (1638, 14) on 37XX (quantization.cpp:344-354)
+    assert (p.mode, p.clamp_low, p.clamp_high, p.lrelu_mult, p.lrelu_shift) == (abi.PPE_LPRELU, 0, 255, 1638, 14)
+    assert p.clamp_domain == abi.CLAMP_POST_ZP
+    # table: ptr = oc * IC*KY*KX, sparsity 0xFFFFFF, word[2] from rescale = w[oc] * in / out, bias 0
+    from oracle import nce_oracle
+    for oc in (0, 17, 47):
+        mult, shift, _ = nce_oracle.quant_approx(((0.004 + 0.0001 * oc) * 0.02) / 0.05)
+        assert list(task.table[oc]) == [oc * 576, 0xFFFFFF, word2(mult, shift), 0]
+    validator.validate(task)
+
+
+def test_unit_test_conv_scale_is_the_known_answer(validator):
+    # rescale 0.01 * 0.01 / 0.01 = 0.01 -> (20971, 21): QuantizationApproximation's documented example
+    case = hwtest.parse(load("zmajor_conv_u8.json"))
+    x, wt, out = buffers(case, np.random.default_rng(2))
+    task = case.build_task(x, wt, out)
+    assert list(task.table[0]) == [0, 0xFFFFFF, word2(20971, 21), 0] and list(task.table[63])[0] == 63 * 256
+    assert task.desc.weights.dtype == abi.DT_U8 and task.desc.weights.zero_point == 0 and task.desc.input.zero_point == 127
+    validator.validate(task)
+
+
+def test_depthwise_pool_and_eltwise_descriptors(validator):
+    rng = np.random.default_rng(3)
+    case = hwtest.parse(load("depthwise_u8.json"))
+    x, wt, out = buffers(case, rng)
+    task = case.build_task(x, wt, out)
+    d, p = task.desc, task._ppe
+    # JSON pad [top, left, bottom, right] = [1, 1, 0, 0]
+    assert (d.kernel_pad_left, d.kernel_pad_right, d.kernel_pad_top, d.kernel_pad_bottom) == (1, 0, 1, 0)
+    assert list(d.weights.dims) == [32, 16, 1, 1] and list(d.kernel_strides) == [2, 2]
+    assert (p.mode, p.clamp_low, p.clamp_high, p.clamp_domain) == (abi.PPE_NOOP, 0 - 128, 255 - 128, abi.CLAMP_PRE_ZP)
+    assert task._variants[0].mpe_mode == abi.MPE_CUBOID_8x16 and task.table.shape == (32, 4) and task.table[5][0] == 5 * 16
+    validator.validate(task)
+
+    case = hwtest.parse(load("maxpool_u8.json"))
+    x, wt, out = buffers(case, rng)
+    task = case.build_task(x, None, out)
+    assert task.table is None and list(task.desc.kernel_size) == [3, 3] and task._ppe.has_quant == 0
+    validator.validate(task)
+
+    case = hwtest.parse(load("avgpool_u8.json"))
+    x, wt, out = buffers(case, rng)
+    task = case.build_task(x, None, out)
+    from oracle import nce_oracle
+    mult, shift, _ = nce_oracle.quant_approx(0.02 / 0.025 / 4.0)
+    p = task._ppe
+    assert task.table is None and (p.has_quant, p.quant_mult, p.quant_shift) == (1, mult, shift)
+    assert (p.clamp_low, p.clamp_high) == (-90, 165)
+    validator.validate(task)
+
+    case = hwtest.parse(load("avgpool_u8_per_channel.json"))
+    task = case.build_task(x, None, out)
+    mult, shift, _ = nce_oracle.quant_approx(((1.0 / 4.0) * 0.02) / (0.02 + 0.0005 * 9))
+    assert task._ppe.has_quant == 0 and list(task.table[9]) == [0, 0xFFFFFF, word2(mult, shift), 0]
+    validator.validate(task)
+
+    case = hwtest.parse(load("eltwise_add_u8.json"))
+    x, wt, out = buffers(case, rng)
+    task = case.build_task(x, wt, out)
+    p = task._ppe
+    # calculateQuantScaleVectorForEltwise: first operand's scale over the output scale: 0.5 -> (16384, 15)
+    assert (p.mode, p.has_quant, p.quant_mult, p.quant_shift, p.has_in_mult) == (abi.PPE_ADD, 1, 16384, 15, 0)
+    assert task.desc.weights.zero_point == 130 and task._variants[0].mpe_mode == abi.MPE_CUBOID_8x16
+    validator.validate(task)
+
+
+def test_what_the_executor_cannot_run_is_reported():
+    d = json.loads(load("zmajor_conv_u8.json"))
+    x = np.zeros((1, 16, 16, 256), np.uint8)
+    cases = [
+        (lambda d: d.update(output_order="nchw"), "ODU permutations"),
+        (lambda d: d["input"][0].update(dtype="fp16"), "not an 8-bit integer type"),
+        (lambda d: d["conv_op"].update(compress=True), "compressed"),
+        (lambda d: d.update(activation={"name": "Mish"}), "unsupported activation"),
+        (lambda d: d["input"][0].pop("quantization"), "quantization parameters are required"),
+    ]
+    ex = nce.Executor(device_id=-1, log_level=1)
+    for mutate, message in cases:
+        dd = json.loads(json.dumps(d))
+        mutate(dd)
+        case = hwtest.parse(json.dumps(dd))
+        with pytest.raises(nce.NCEError) as e:
+            case.build_task(x, np.zeros((64, 1, 1, 256), np.uint8), np.zeros((1, 16, 16, 64), np.uint8), executor=ex)
+        assert e.value.code == abi.ERROR_UNSUPPORTED and message in e.value.log, e.value.log
+
+
+# ---- execution ---------------------------------------------------------------------------------------
+
+ALL = ["zmajor_conv_u8.json", "zmajor_conv3x3_lrelu_per_channel.json", "depthwise_u8.json", "maxpool_u8.json",
+       "avgpool_u8.json", "avgpool_u8_per_channel.json", "eltwise_add_u8.json"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ALL)
+def test_descriptors_run_bit_exact(executor, name):
+    import torch
+    from oracle import nce_oracle
+    case = hwtest.parse(load(name))
+    x, wt, out = buffers(case, np.random.default_rng(11))
+    want = out.copy()
+    nce_oracle.run(case.build_task(x, wt, want))
+    dx = torch.from_numpy(x).cuda()
+    dw = torch.from_numpy(wt).cuda() if wt is not None else None
+    dout = torch.full(out.shape, 0x5A, dtype=torch.uint8, device="cuda")
+    task = case.build_task(dx, dw, dout, executor=executor)
+    stream = torch.cuda.current_stream().cuda_stream
+    executor.enqueue(task, stream)
+    executor.synchronize(stream)
+    got = dout.cpu().numpy()
+    assert want.std() > 1.0, "degenerate expected output"
+    assert np.array_equal(got, want)
