@@ -87,7 +87,9 @@ typedef enum nce_clamp_domain_t { NCE_CLAMP_POST_ZP = 0, NCE_CLAMP_PRE_ZP = 1 } 
  * (src/vpux_compiler/src/dialect/VPUIP/ops/nce_cluster_task.cpp:346-359,418-433,702-709): NHWC for
  * activations and OYXI for conv weights, i.e. the C / IC dimension is innermost and must be compact
  * (strides_bytes[1] == element size). The other strides are free, which is how parent_input /
- * parent_output sub-views are expressed. */
+ * parent_output sub-views are expressed. The OUTPUT of a task may instead use any non-overlapping strides,
+ * channel stride included: that is how the ODU permutations (output written as NWHC, NWCH, NCWH, NHCW or NCHW,
+ * getODUPermutationType, nce_cluster_task.cpp:764-780) are expressed; such outputs are written byte by byte. */
 typedef struct nce_tensor_t {
     void* data;
     int32_t dtype;      /* nce_dtype_t */

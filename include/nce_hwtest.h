@@ -78,13 +78,14 @@ nce_result_t nceHwtestGetCase(nce_hwtest_case_handle_t hw_case, nce_hwtest_case_
 nce_result_t nceHwtestGetScales(nce_hwtest_case_handle_t hw_case, int32_t which, double* scales, int32_t capacity);
 
 /* Fill a task the way the case's builder does. On return `desc` holds task type, dtypes, zero points, logical
- * dims and DENSE NHWC / OYXI strides (data pointers NULL: the caller sets them), kernel / stride / pad, one
+ * dims and DENSE strides (inputs NHWC, weights OYXI, output in the case's output_order; data pointers NULL: the
+ * caller sets them), kernel / stride / pad, one
  * whole-output variant in `variant` and the PPE attributes in `ppe` (desc->variants / desc->ppe point at them).
  * `table` receives OC rows of 4 int32 when the builder emits a weights table (CONV, DWCONV; pools / eltwise only
  * for per-channel output scales); *table_rows tells how many rows were written (0 = no table).
  * Depthwise weights are described in their padded memory form [C, 16 * ceil(KY*KX / 16)].
- * Returns NCE_RESULT_ERROR_UNSUPPORTED for case types, data types, activations or output orders the executor
- * cannot run (the log names which). */
+ * Returns NCE_RESULT_ERROR_UNSUPPORTED for case types, data types or activations the executor cannot run (the log
+ * names which). */
 nce_result_t nceHwtestBuildTask(nce_hwtest_case_handle_t hw_case, nce_cluster_task_desc_t* desc, nce_dpu_task_t* variant,
                                 nce_ppe_task_t* ppe, int32_t* table, int32_t table_capacity_rows, int32_t* table_rows,
                                 nce_log_handle_t log);

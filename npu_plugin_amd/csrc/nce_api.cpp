@@ -59,18 +59,40 @@ int64_t clamp64(int64_t v, int64_t lo, int64_t hi) {
 
 // Activation tensor: NHWC, channels compact and a multiple of 16 for 8-bit types
 // (nce_cluster_task.cpp:346-359,702-709; src/vpux_compiler/src/dialect/VPU/utils/nce_invariant.cpp:135-153).
-nce_result_t check_activation(nce_log_s* log, const char* name, const nce_tensor_t& x, TensorDev* out) {
+// An OUTPUT may instead be laid out in any order of H, W, C under N - the ODU permutations NWHC, NWCH, NCWH,
+// NHCW, NCHW (getODUPermutationType, nce_cluster_task.cpp:764-780) - expressed through its strides: any
+// non-overlapping strides are accepted and written byte by byte.
+nce_result_t check_activation(nce_log_s* log, const char* name, const nce_tensor_t& x, TensorDev* out, bool allow_permuted = false) {
     if (x.data == nullptr) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: data pointer is null", name);
     if (!is_8bit(x.dtype)) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: only u8 / i8 storage is supported, got dtype %d", name, x.dtype);
     for (int i = 0; i < 4; ++i)
         if (x.dims[i] <= 0 || x.dims[i] > 0x7fffffff) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: dims[%d] = %lld", name, i, (long long)x.dims[i]);
     if (x.dims[1] % 16 != 0) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: channels (%lld) must be a multiple of 16", name, (long long)x.dims[1]);
-    if (x.strides_bytes[1] != 1) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: layout must be NHWC with compact channels (C stride %lld)", name, (long long)x.strides_bytes[1]);
-    if (x.strides_bytes[3] < x.dims[1] || x.strides_bytes[2] < x.strides_bytes[3] * 1 || x.strides_bytes[0] < x.strides_bytes[2])
-        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides are not NHWC-ordered (N %lld, H %lld, W %lld, C 1)", name,
-             (long long)x.strides_bytes[0], (long long)x.strides_bytes[2], (long long)x.strides_bytes[3]);
-    if (((uintptr_t)x.data | (uintptr_t)x.strides_bytes[0] | (uintptr_t)x.strides_bytes[2] | (uintptr_t)x.strides_bytes[3]) & 15)
-        FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
+    if (allow_permuted) {
+        int order[4] = {0, 1, 2, 3};
+        std::sort(order, order + 4, [&](int l, int r) { return x.strides_bytes[l] < x.strides_bytes[r]; });
+        int64_t need = 1;
+        for (int i = 0; i < 4; ++i) {
+            const int d = order[i];
+            if (x.dims[d] == 1) continue;  // the stride of an extent-1 dimension is never used
+            if (x.strides_bytes[d] < need)
+                FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides (N %lld, C %lld, H %lld, W %lld) make elements overlap", name,
+                     (long long)x.strides_bytes[0], (long long)x.strides_bytes[1], (long long)x.strides_bytes[2], (long long)x.strides_bytes[3]);
+            need = x.strides_bytes[d] * x.dims[d];
+        }
+        if (need > 0x7fffffff00LL) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: tensor too large", name);
+        // compact channels are written with 128-bit stores
+        if (x.strides_bytes[1] == 1 &&
+            (((uintptr_t)x.data | (uintptr_t)x.strides_bytes[0] | (uintptr_t)x.strides_bytes[2] | (uintptr_t)x.strides_bytes[3]) & 15))
+            FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
+    } else {
+        if (x.strides_bytes[1] != 1) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: layout must be NHWC with compact channels (C stride %lld)", name, (long long)x.strides_bytes[1]);
+        if (x.strides_bytes[3] < x.dims[1] || x.strides_bytes[2] < x.strides_bytes[3] * 1 || x.strides_bytes[0] < x.strides_bytes[2])
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides are not NHWC-ordered (N %lld, H %lld, W %lld, C 1)", name,
+                 (long long)x.strides_bytes[0], (long long)x.strides_bytes[2], (long long)x.strides_bytes[3]);
+        if (((uintptr_t)x.data | (uintptr_t)x.strides_bytes[0] | (uintptr_t)x.strides_bytes[2] | (uintptr_t)x.strides_bytes[3]) & 15)
+            FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
+    }
     int64_t lo, hi;
     type_range(x.dtype, &lo, &hi);
     if (x.zero_point < lo || x.zero_point > hi) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: zero point %d outside the storage range", name, x.zero_point);
@@ -78,6 +100,7 @@ nce_result_t check_activation(nce_log_s* log, const char* name, const nce_tensor
     out->sn = x.strides_bytes[0];
     out->sh = x.strides_bytes[2];
     out->sw = x.strides_bytes[3];
+    out->sc = x.strides_bytes[1];
     out->n = (int32_t)x.dims[0];
     out->c = (int32_t)x.dims[1];
     out->h = (int32_t)x.dims[2];
@@ -284,7 +307,7 @@ nce_result_t make_plan(nce_log_s* log, const nce_cluster_task_desc_t* t, Plan* p
     }
     nce_result_t r;
     if ((r = check_activation(log, "input", t->input, &d.in)) != NCE_RESULT_SUCCESS) return r;
-    if ((r = check_activation(log, "output", t->output, &d.out)) != NCE_RESULT_SUCCESS) return r;
+    if ((r = check_activation(log, "output", t->output, &d.out, true)) != NCE_RESULT_SUCCESS) return r;
 
     const bool has_table = t->weight_table.data != nullptr;
     if (has_table && (r = check_table(log, t->weight_table, d.out.c, &d)) != NCE_RESULT_SUCCESS) return r;

@@ -31,7 +31,8 @@ struct Box {
 
 struct TensorDev {
     uint8_t* data;
-    int64_t sn, sh, sw;  // strides in bytes for N, H, W (C is compact)
+    int64_t sn, sh, sw;  // strides in bytes for N, H, W
+    int64_t sc;          // channel stride: 1 (NHWC) except for outputs in a permuted order (ODU permutation)
     int32_t n, c, h, w;
     int32_t is_signed;   // storage type i8
     int32_t zp;
@@ -59,6 +60,27 @@ __host__ __device__ inline uint32_t xcd_grid(uint32_t ntiles) {
 __device__ inline uint32_t xcd_tile(uint32_t block_id, uint32_t ntiles) {
     const uint32_t per_xcd = (ntiles + kNumXcd - 1) / kNumXcd;
     return (block_id % kNumXcd) * per_xcd + block_id / kNumXcd;
+}
+
+// Store 16 (or 8) consecutive channels of one pixel: one vector store when channels are compact, byte
+// stores at the channel stride for permuted output orders. p points at the first of those channels.
+__device__ __forceinline__ void store_channels16(uint8_t* p, int64_t sc, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+    if (sc == 1) {
+        *reinterpret_cast<uint4*>(p) = make_uint4(w0, w1, w2, w3);
+    } else {
+        const uint32_t w[4] = {w0, w1, w2, w3};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) p[i * sc] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+    }
+}
+__device__ __forceinline__ void store_channels8(uint8_t* p, int64_t sc, uint32_t w0, uint32_t w1) {
+    if (sc == 1) {
+        *reinterpret_cast<uint2*>(p) = make_uint2(w0, w1);
+    } else {
+        const uint32_t w[2] = {w0, w1};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) p[i * sc] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+    }
 }
 
 hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);

@@ -210,7 +210,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
         const int32_t bx = pp - rr * a.bw;
         const int32_t n = fdiv(rr, a.div_bh);
         const int32_t by = rr - n * a.bh;
-        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0 * a.out_sc;
         a_corr[x] = a.dw != 0 ? a.dw * (sAsum[prow] + a.ktot * a.da) : 0;
     }
     if (a.dw != 0) epi_store<2, PXF, true>(a, es, acc, 0, noc, half, dst, p_valid, a_corr, mode, pu);
@@ -251,6 +251,7 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.out_sn = t.out.sn;
     a.out_sh = t.out.sh;
     a.out_sw = t.out.sw;
+    a.out_sc = t.out.sc;
     a.x0 = box.x0;
     a.y0 = box.y0;
     a.z0 = box.z0;

@@ -41,7 +41,7 @@ struct ConvArgs {
     const int32_t* table;
     int64_t table_stride;
     uint8_t* out;
-    int64_t out_sn, out_sh, out_sw;
+    int64_t out_sn, out_sh, out_sw, out_sc;
     int32_t x0, y0, z0, bw, bh, bc;
     int32_t M;  // pixels in the box over all batches (< 2^31)
     FastDiv div_bw, div_bh, div_pitch, div_rows_full;
@@ -178,7 +178,7 @@ __device__ __forceinline__ void epi_store_mode(const ConvArgs& a, const EpiSmem&
         }
 #pragma unroll
         for (int x = 0; x < BF; ++x)
-            if (valid[x]) *reinterpret_cast<uint4*>(dst[x] + ocl) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
+            if (valid[x]) store_channels16(dst[x] + ocl * a.out_sc, a.out_sc, wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
     }
 }
 

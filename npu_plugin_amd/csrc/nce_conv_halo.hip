@@ -256,7 +256,7 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     for (int x = 0; x < BF; ++x) {
         const int32_t n = fdiv(b_rr[x], a.div_bh);
         const int by = b_rr[x] - n * a.bh;
-        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + b_bx[x]) * a.out_sw + oc0;
+        dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + b_bx[x]) * a.out_sw + oc0 * a.out_sc;
         acorr[x] = 0;
     }
     epi_store<AF, BF, false>(a, es, acc, wn * AF * 32, noc, half, dst, valid, acorr, mode, pu);

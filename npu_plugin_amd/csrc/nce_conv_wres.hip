@@ -150,8 +150,8 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
 #pragma unroll
     for (int x = 0; x < BF; ++x) {
         if (!valid[x]) continue;
-        if constexpr (NF == 4) *reinterpret_cast<uint4*>(dst[x] + ch0) = make_uint4(wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
-        else *reinterpret_cast<uint2*>(dst[x] + ch0) = make_uint2(wo[x][0], wo[x][1]);
+        if constexpr (NF == 4) store_channels16(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
+        else store_channels8(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1]);
     }
 }
 
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t iy0 = (a.y0 + by) * a.SY - a.PT;
             const int32_t ix0 = (a.x0 + bx) * a.SX - a.PL;
             pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + (MODE == WRES_GENERIC ? 0 : q * 16);
-            dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0;
+            dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0 * a.out_sc;
             mask0[x] = mask1[x] = 0;
             if (MODE != WRES_FAST) {
                 const uint32_t rows = bit_range(max(0, -iy0), min(a.KY, a.H - iy0));

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
             const int64_t y = box.y0 + by, x = box.x0 + bx;
             off_a = n * t.in.sn + y * t.in.sh + x * t.in.sw + oc;
             off_b = n * t.in2.sn + y * t.in2.sh + x * t.in2.sw + oc;
-            off_o = n * t.out.sn + y * t.out.sh + x * t.out.sw + oc;
+            off_o = n * t.out.sn + y * t.out.sh + x * t.out.sw + oc * t.out.sc;
         }
         const uint4 va = *reinterpret_cast<const uint4*>(t.in.data + off_a);
         const uint4 vb = *reinterpret_cast<const uint4*>(t.in2.data + off_b);
@@ -80,12 +80,12 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
             }
             wo[d] = packed;
         }
-        *reinterpret_cast<uint4*>(t.out.data + off_o) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+        store_channels16(t.out.data + off_o, FLAT ? 1 : t.out.sc, wo[0], wo[1], wo[2], wo[3]);
     }
 }
 
 bool is_dense_nhwc(const TensorDev& x) {
-    return x.sw == x.c && x.sh == (int64_t)x.w * x.c && x.sn == (int64_t)x.h * x.w * x.c;
+    return x.sc == 1 && x.sw == x.c && x.sh == (int64_t)x.w * x.c && x.sn == (int64_t)x.h * x.w * x.c;
 }
 
 template <bool FLAT, int PATH>

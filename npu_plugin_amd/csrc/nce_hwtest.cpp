@@ -583,8 +583,6 @@ void build(const nce_hwtest_case_s& c, nce_cluster_task_desc_t* d, nce_dpu_task_
     need_quant8(c.in, "input");
     need_quant8(c.out, "output");
     if (c.in.scales.size() != 1) throw Unsupported("input: per-channel activation scales are not supported");
-    if (strcmp(p.output_order, "nhwc") != 0)
-        throw Unsupported(std::string("output_order '") + p.output_order + "': ODU permutations are not implemented");
     const int64_t N = p.input.shape[0], IC = p.input.shape[1], IH = p.input.shape[2], IW = p.input.shape[3];
     const int64_t OC = p.output.shape[1], OH = p.output.shape[2], OW = p.output.shape[3];
     if (p.output.shape[0] != N) throw std::runtime_error("output batch differs from input batch");
@@ -596,6 +594,17 @@ void build(const nce_hwtest_case_s& c, nce_cluster_task_desc_t* d, nce_dpu_task_
     d->task_type = p.task_type;
     dense_nhwc(&d->input, p.input.dtype, N, IC, IH, IW, p.input.zero_point);
     dense_nhwc(&d->output, p.output.dtype, N, OC, OH, OW, p.output.zero_point);
+    {   // ODU permutation: the output is dense in the order "output_order" names, outermost first
+        // (oduPermutationToLayout, hwtest_utils.cpp; getODUPermutationType, nce_cluster_task.cpp:764-780)
+        int64_t stride = 1;
+        for (int i = 3; i >= 1; --i) {
+            const char dim = p.output_order[i];
+            const int idx = dim == 'c' ? 1 : dim == 'h' ? 2 : 3;
+            d->output.strides_bytes[idx] = stride;
+            stride *= d->output.dims[idx];
+        }
+        d->output.strides_bytes[0] = stride;
+    }
     d->weights.dtype = NCE_DT_U8;
     d->weight_table.dtype = NCE_DT_SI32;
     // JSON pads are [top, left, bottom, right] (hwtest_utils.hpp:24-35, convertNBPadtoNCETaskPad hwtest_utils.cpp:218-227)

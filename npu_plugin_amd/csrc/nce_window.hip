@@ -151,7 +151,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         const int32_t oy = box.y0 + by, ox = box.x0 + bx;
         const int32_t iy0 = oy * t.sy - t.pt, ix0 = ox * t.sx - t.pl;
         const uint8_t* src = t.in.data + n * t.in.sn + oc;
-        uint8_t* dst = t.out.data + n * t.out.sn + (int64_t)oy * t.out.sh + (int64_t)ox * t.out.sw + oc;
+        uint8_t* dst = t.out.data + n * t.out.sn + (int64_t)oy * t.out.sh + (int64_t)ox * t.out.sw + oc * t.out.sc;
 
         if (MODE == MODE_MAX) {
             // even / odd bytes of each dword as packed u16; order-preserving re-bias for i8
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 const uint32_t o = pk_min_u16(pk_max_u16(mo[d], lo2), hi2);
                 wo[d] = (e | (o << 8)) ^ a.a_xor;
             }
-            *reinterpret_cast<uint4*>(dst) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+            store_channels16(dst, t.out.sc, wo[0], wo[1], wo[2], wo[3]);
             continue;
         }
 
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
             }
         }
-        *reinterpret_cast<uint4*>(dst) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+        store_channels16(dst, t.out.sc, wo[0], wo[1], wo[2], wo[3]);
     }
 }
 

@@ -333,7 +333,7 @@ typedef struct {
     uint8_t* out;
     int64_t is_n, is_h, is_w;   /* input strides (bytes) */
     int64_t ws_n, ws_h, ws_w;   /* weights / second-input strides */
-    int64_t os_n, os_h, os_w;   /* output strides */
+    int64_t os_n, os_h, os_w, os_c;   /* output strides (os_c != 1: permuted output order) */
     int64_t tab_stride;         /* int32 elements between table rows */
 } ctx_t;
 
@@ -356,7 +356,7 @@ static int32_t scale_for(const ctx_t* c, int64_t oc, int32_t* mult, int32_t* shi
  * 32-bit hardware accumulator. */
 static void eval_element(const ctx_t* c, int64_t n, int64_t oy, int64_t ox, int64_t oc) {
     const nce_cluster_task_desc_t* t = c->t;
-    uint8_t* dst = c->out + n * c->os_n + oy * c->os_h + ox * c->os_w + oc;
+    uint8_t* dst = c->out + n * c->os_n + oy * c->os_h + ox * c->os_w + oc * c->os_c;
     int64_t acc = 0;
     switch (t->task_type) {
     case NCE_TASK_CONV: {
@@ -486,9 +486,10 @@ int nce_oracle_run(const nce_cluster_task_desc_t* t, int nthreads) {
     c.os_n = t->output.strides_bytes[0];
     c.os_h = t->output.strides_bytes[2];
     c.os_w = t->output.strides_bytes[3];
+    c.os_c = t->output.strides_bytes[1];
     c.table = (const int32_t*)t->weight_table.data;
     c.tab_stride = c.table ? t->weight_table.strides_bytes[0] / 4 : 0;
-    if (t->input.strides_bytes[1] != 1 || t->output.strides_bytes[1] != 1) return -2;
+    if (t->input.strides_bytes[1] != 1) return -2;
     if (t->output.dims[0] != c.N) return -2;
 
     switch (t->task_type) {

@@ -370,3 +370,56 @@ def test_conv_gather_kernel_shapes(executor, gather_path, shape):
 def test_conv_wide_kernel_falls_back(executor):
     # 7x7 with 64 input channels needs more than 31 tap bits: the halo / gather kernels take it
     check(K.conv_case(511, 1, 20, 20, 64, 32, k=(7, 7), s=(1, 1), pads=(3, 3, 3, 3), in_zp=100), executor)
+
+
+# ---- ODU permutation: outputs written in any order of H, W, C ----------------------------------------
+
+ODU_ORDERS = {"nhwc": (0, 1, 2, 3), "nwhc": (0, 2, 1, 3), "nwch": (0, 2, 3, 1), "ncwh": (0, 3, 2, 1),
+              "nhcw": (0, 1, 3, 2), "nchw": (0, 3, 1, 2)}   # memory order as axes of the (N, H, W, C) result
+
+
+def _permuted_run(case, order, executor):
+    """Runs the case with its output laid out in `order`; returns (hip, oracle) as (N, H, W, C) arrays."""
+    import torch
+    from oracle import nce_oracle
+    axes = ODU_ORDERS[order]
+    inverse = [axes.index(i) for i in range(4)]
+    mem_shape = tuple(case.out_shape[a] for a in axes)
+    host = np.full(mem_shape, 0x5A, dtype=np.uint8)
+    nce_oracle.run(K.build_task(case, case.input, case.weights, case.table, host.transpose(inverse)))
+    dc = K.DeviceCase(case)
+    dev = torch.full(mem_shape, 0x5A, dtype=torch.uint8, device="cuda")
+    task = K.build_task(case, dc.input, dc.weights, dc.table, dev.permute(*inverse))
+    stream = torch.cuda.current_stream().cuda_stream
+    executor.enqueue(task, stream)
+    executor.synchronize(stream)
+    return dev.cpu().numpy().transpose(inverse), host.transpose(inverse)
+
+
+@pytest.mark.parametrize("order", list(ODU_ORDERS))
+def test_odu_permutation_conv(executor, order):
+    case = K.conv_case(600, 2, 11, 13, 64, 48, in_zp=99,
+                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14))
+    got, want = _permuted_run(case, order, executor)
+    assert np.array_equal(want, K.run_oracle(case)), "the oracle itself must be layout-independent"
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("order", ["nchw", "nwch", "nhcw"])
+def test_odu_permutation_other_tasks(executor, order, monkeypatch):
+    cases = [K.conv_case(601, 1, 9, 9, 16, 32, k=(5, 5), pads=(2, 2, 2, 2)),            # per-lane tap path
+             K.dw_case(602, 2, 13, 13, 32), K.pool_case(603, True, 2, 12, 12, 32), K.pool_case(604, False, 2, 12, 12, 32),
+             K.eltwise_case(605, 2, 9, 7, 48)]
+    for case in cases:
+        got, want = _permuted_run(case, order, executor)
+        assert np.array_equal(got, want), case.name
+    for path in ("1", "2"):  # halo and gather kernels
+        monkeypatch.setenv("NCE_HIP_CONV_PATH", path)
+        got, want = _permuted_run(K.conv_case(606, 2, 10, 10, 64, 64), order, executor)
+        assert np.array_equal(got, want), f"conv path {path}"
+
+
+def test_odu_permutation_variants_leave_other_bytes_alone(executor):
+    case = K.conv_case(607, 1, 12, 12, 64, 64, variants=[((2, 3, 16), (9, 10, 47))])
+    got, want = _permuted_run(case, "nchw", executor)
+    assert np.array_equal(got, want) and (want == 0x5A).sum() > want.size // 2

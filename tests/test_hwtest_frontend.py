@@ -93,7 +93,8 @@ def buffers(case, rng):
     i, w, o = case.info.input, case.info.weight, case.info.output
     n, c, h, wd = i.shape
     x = rng.integers(0, 256, (n, h, wd, c), dtype=np.uint8)
-    out = np.zeros((o.shape[0], o.shape[2], o.shape[3], o.shape[1]), dtype=np.uint8)
+    extent = {"n": o.shape[0], "c": o.shape[1], "h": o.shape[2], "w": o.shape[3]}
+    out = np.zeros([extent[d] for d in case.output_order], dtype=np.uint8)   # dense in the case's output order
     wt = None
     if case.task_type == abi.TASK_CONV:
         dt = np.int8 if w.dtype == abi.DT_I8 else np.uint8
@@ -188,7 +189,6 @@ def test_what_the_executor_cannot_run_is_reported():
     d = json.loads(load("zmajor_conv_u8.json"))
     x = np.zeros((1, 16, 16, 256), np.uint8)
     cases = [
-        (lambda d: d.update(output_order="nchw"), "ODU permutations"),
         (lambda d: d["input"][0].update(dtype="fp16"), "not an 8-bit integer type"),
         (lambda d: d["conv_op"].update(compress=True), "compressed"),
         (lambda d: d.update(activation={"name": "Mish"}), "unsupported activation"),
@@ -206,7 +206,23 @@ def test_what_the_executor_cannot_run_is_reported():
 
 # ---- execution ---------------------------------------------------------------------------------------
 
-ALL = ["zmajor_conv_u8.json", "zmajor_conv3x3_lrelu_per_channel.json", "depthwise_u8.json", "maxpool_u8.json",
+def test_output_order_becomes_output_strides(validator):
+    case = hwtest.parse(load("zmajor_conv3x3_output_nchw.json"))
+    x, wt, out = buffers(case, np.random.default_rng(4))
+    assert out.shape == (1, 48, 18, 18)
+    task = case.build_task(x, wt, out)
+    assert list(task.desc.output.dims) == [1, 48, 18, 18] and list(task.desc.output.strides_bytes) == [48 * 324, 324, 18, 1]
+    validator.validate(task)
+    # same bytes as the nhwc run, transposed
+    from oracle import nce_oracle
+    nce_oracle.run(task)
+    ref_case = hwtest.parse(load("zmajor_conv3x3_lrelu_per_channel.json"))
+    ref = np.zeros((1, 18, 18, 48), dtype=np.uint8)
+    nce_oracle.run(ref_case.build_task(x, wt, ref))
+    assert ref.std() > 1.0 and np.array_equal(out.transpose(0, 2, 3, 1), ref)
+
+
+ALL = ["zmajor_conv_u8.json", "zmajor_conv3x3_lrelu_per_channel.json", "zmajor_conv3x3_output_nchw.json", "depthwise_u8.json", "maxpool_u8.json",
        "avgpool_u8.json", "avgpool_u8_per_channel.json", "eltwise_add_u8.json"]
 
 

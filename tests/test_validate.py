@@ -187,6 +187,21 @@ def test_zero_point_ranges(validator):
     assert code(validator, task_of(c))[0] == abi.ERROR_INVALID_ARGUMENT
 
 
+def test_permuted_output_strides(validator):
+    # ODU permutation: the output (only) may use any non-overlapping strides
+    c = K.cfg1()
+    out = np.zeros((1, 16, 32, 32), dtype=np.uint8)                    # NCHW memory
+    task = K.build_task(c, c.input, c.weights, c.table, out.transpose(0, 2, 3, 1))
+    assert task.desc.output.strides_bytes[1] == 1024
+    validator.validate(task)
+    overlapping = np.lib.stride_tricks.as_strided(out, shape=(1, 32, 32, 16), strides=(16384, 32, 1, 16))
+    assert code(validator, K.build_task(c, c.input, c.weights, c.table, overlapping))[0] == abi.ERROR_INVALID_ARGUMENT
+    # the input must stay NHWC
+    x = np.ascontiguousarray(c.input.transpose(0, 3, 1, 2)).transpose(0, 2, 3, 1)
+    r = code(validator, K.build_task(c, x, c.weights, c.table, np.zeros(c.out_shape, np.uint8)))
+    assert r[0] == abi.ERROR_INVALID_ARGUMENT and "compact channels" in r[1]
+
+
 def test_log_two_call_pattern(validator):
     lib = abi.load_library()
     t = task_of(K.cfg1())
