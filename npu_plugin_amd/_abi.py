@@ -1,4 +1,4 @@
-"""ctypes view of include/nce_hip.h, nce_params.h and nce_hwtest.h, and the loader of libnce_hip.so.
+"""ctypes view of include/nce_hip.h, nce_params.h, nce_hwtest.h and nce_vpuip.h, and the loader of libnce_hip.so.
 
 The shared library is the product: loading fails loudly when it has not been built, and nothing
 here falls back to a CPU implementation.
@@ -159,6 +159,30 @@ class HwtestCase(C.Structure):
     ]
 
 
+class VpuipBuffer(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 32),
+        ("section", C.c_int32),
+        ("index", C.c_int32),
+        ("byte_offset", C.c_int64),
+        ("byte_size", C.c_int64),
+        ("dtype", C.c_int32),
+        ("elem_bytes", C.c_int32),
+        ("zero_point", C.c_int32),
+        ("dims", C.c_int64 * 4),
+        ("strides_bytes", C.c_int64 * 4),
+    ]
+
+
+class VpuipInfo(C.Structure):
+    _fields_ = [("num_buffers", C.c_int32), ("num_ops", C.c_int32), ("num_tasks", C.c_int32), ("num_dmas", C.c_int32),
+                ("function", C.c_char * 64)]
+
+
+# nce_vpuip_section_t / nce_vpuip_op_kind_t
+VPUIP_ARGUMENT, VPUIP_CMX_NN, VPUIP_DDR, VPUIP_NETWORK_INPUT, VPUIP_NETWORK_OUTPUT = range(5)
+VPUIP_OP_NCE_TASK, VPUIP_OP_DMA = 0, 1
+
 # nce_hwtest_activation_t
 HWTEST_ACT_NONE, HWTEST_ACT_RELU, HWTEST_ACT_RELUX, HWTEST_ACT_LEAKY_RELU, HWTEST_ACT_OTHER = range(5)
 
@@ -187,6 +211,14 @@ SYMBOLS = {
     "nceHwtestDestroy": (C.c_int, [C.c_void_p]),
     "nceHwtestGetCase": (C.c_int, [C.c_void_p, _P(HwtestCase)]),
     "nceHwtestGetScales": (C.c_int, [C.c_void_p, C.c_int32, _P(C.c_double), C.c_int32]),
+    "nceVpuipParse": (C.c_int, [C.c_char_p, _P(C.c_void_p), C.c_void_p]),
+    "nceVpuipDestroy": (C.c_int, [C.c_void_p]),
+    "nceVpuipGetInfo": (C.c_int, [C.c_void_p, _P(VpuipInfo)]),
+    "nceVpuipGetBuffer": (C.c_int, [C.c_void_p, C.c_int32, _P(VpuipBuffer)]),
+    "nceVpuipGetOp": (C.c_int, [C.c_void_p, C.c_int32, _P(C.c_int32), _P(C.c_int32)]),
+    "nceVpuipBind": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_int64]),
+    "nceVpuipGetTask": (C.c_int, [C.c_void_p, C.c_int32, _P(ClusterTaskDesc), C.c_void_p]),
+    "nceVpuipEnqueue": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "nceHwtestBuildTask": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc), _P(DpuTask), _P(PpeTask), _P(C.c_int32), C.c_int32,
                                      _P(C.c_int32), C.c_void_p]),
 }

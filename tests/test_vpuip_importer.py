@@ -1,0 +1,148 @@
+"""Importer of VPUIP programs in textual form (include/nce_vpuip.h)."""
+import os
+
+import numpy as np
+import pytest
+
+import npu_plugin_amd as nce
+from npu_plugin_amd import _abi as abi
+from npu_plugin_amd import vpuip
+from tests import cases as K
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vpuip")
+TEXT = open(os.path.join(GOLDEN, "conv_then_add_u8.mlir")).read()
+
+
+def test_buffers_types_and_program_order():
+    prog = vpuip.parse(TEXT)
+    assert prog.function == "convThenAdd" and prog.num_tasks == 2 and prog.num_dmas == 4
+    assert [k for k, _ in prog.ops] == [abi.VPUIP_OP_DMA] * 3 + [abi.VPUIP_OP_NCE_TASK] * 2 + [abi.VPUIP_OP_DMA]
+    arg0, w, table, mid = prog.buffer("%arg0"), prog.buffer("%1"), prog.buffer("%2"), prog.buffer("%3")
+    assert (arg0.section, arg0.index, arg0.dtype, arg0.zero_point) == (vpuip.ARGUMENT, 0, abi.DT_U8, 128)
+    assert list(arg0.dims) == [1, 32, 12, 12] and list(arg0.strides_bytes) == [4608, 1, 384, 32]      # NHWC
+    assert (w.section, w.index, w.byte_offset, w.byte_size, w.zero_point) == (vpuip.CMX_NN, 0, 4608, 9216, 127)
+    assert list(w.dims) == [32, 32, 3, 3] and list(w.strides_bytes) == [288, 1, 96, 32]                 # OYXI
+    assert (table.dtype, table.elem_bytes, table.byte_size) == (abi.DT_SI32, 4, 512) and list(table.strides_bytes)[0] == 16
+    assert mid.zero_point == 121 and prog.buffer("%6").section == vpuip.DDR
+    assert prog.section_size(vpuip.CMX_NN, 0) == 18944 + 4608 and prog.section_size(vpuip.DDR, 0) == 9216 + 512
+
+
+def test_task_descriptors(validator):
+    prog = vpuip.parse(TEXT)
+    cmx = np.zeros(prog.section_size(vpuip.CMX_NN, 0), dtype=np.uint8)
+    prog.bind(vpuip.CMX_NN, 0, cmx)
+    conv = prog.task(0).desc
+    assert conv.task_type == abi.TASK_CONV and list(conv.kernel_size) == [3, 3] and list(conv.kernel_strides) == [1, 1]
+    assert (conv.kernel_pad_left, conv.kernel_pad_right, conv.kernel_pad_top, conv.kernel_pad_bottom) == (1, 1, 1, 1)
+    assert conv.num_variants == 2 and list(conv.variants[1].out_start) == [0, 6, 0] and list(conv.variants[1].out_end) == [11, 11, 31]
+    assert (conv.variants[0].pad_top, conv.variants[0].pad_bottom, conv.variants[1].pad_top, conv.variants[1].pad_bottom) == (1, 0, 0, 1)
+    p = conv.ppe.contents
+    assert (p.mode, p.clamp_low, p.clamp_high, p.lrelu_mult, p.lrelu_shift, p.has_quant) == (abi.PPE_LPRELU, 0, 255, 1638, 14, 0)
+    assert conv.input.data == cmx.ctypes.data and conv.weights.data == cmx.ctypes.data + 4608
+    assert conv.weights.dtype == abi.DT_U8 and conv.weights.zero_point == 127 and conv.output.zero_point == 121
+    add = prog.task(1).desc
+    p = add.ppe.contents
+    assert add.task_type == abi.TASK_ELTWISE and add.variants[0].mpe_mode == abi.MPE_CUBOID_8x16
+    assert (p.mode, p.has_quant, p.quant_mult, p.quant_shift, p.has_in_mult, p.in1_quant_mult, p.in2_quant_mult) == \
+        (abi.PPE_ADD, 1, 25600, 30, 1, 20480, 8192)
+    assert (p.clamp_low, p.clamp_high) == (3, 255) and add.weights.zero_point == 128 and add.output.zero_point == 3
+    validator.validate(prog.task(0))
+    validator.validate(prog.task(1))
+
+
+def _reference_result(x, wt, table):
+    """The same two tasks built by hand and evaluated by the oracle."""
+    from oracle import nce_oracle
+    conv = K.Case("conv", nce.TASK_CONV, x, (1, 12, 12, 32), 128, 121, False, wt, 127, table, (3, 3), (1, 1), (1, 1, 1, 1),
+                  dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14), None)
+    mid = np.zeros((1, 12, 12, 32), np.uint8)
+    nce_oracle.run(K.build_task(conv, x, wt, table, mid))
+    add = K.Case("add", nce.TASK_ELTWISE, mid, (1, 12, 12, 32), 121, 3, False, x, 128, None, None, None, (0, 0, 0, 0),
+                 dict(mode=nce.PPE_ADD, clamp_low=3, clamp_high=255, quant_mult=25600, quant_shift=30, in1_quant_mult=20480,
+                      in2_quant_mult=8192), None)
+    out = np.zeros((1, 12, 12, 32), np.uint8)
+    nce_oracle.run(K.build_task(add, mid, x, None, out))
+    return mid, out
+
+
+def _operands(seed=5):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, (1, 12, 12, 32), dtype=np.uint8)
+    wt = rng.integers(0, 255, (32, 3, 3, 32), dtype=np.uint8)
+    table = K.make_table(rng, 32, 288, 2e-3, 8e-3, 500.0)
+    return x, wt, table
+
+
+def test_tasks_from_the_program_match_hand_built_tasks_on_the_oracle():
+    from oracle import nce_oracle
+    prog = vpuip.parse(TEXT)
+    x, wt, table = _operands()
+    cmx = np.zeros(prog.section_size(vpuip.CMX_NN, 0), dtype=np.uint8)
+    cmx[0:4608] = x.ravel()                                   # what the three input DMAs would have copied
+    cmx[4608:13824] = wt.ravel()
+    cmx[13824:14336] = table.view(np.uint8).ravel()
+    prog.bind(vpuip.CMX_NN, 0, cmx)
+    nce_oracle.run(prog.task(0))
+    nce_oracle.run(prog.task(1))
+    mid, out = _reference_result(x, wt, table)
+    assert mid.std() > 5 and out.std() > 5
+    assert np.array_equal(cmx[14336:18944].reshape(mid.shape), mid)
+    assert np.array_equal(cmx[18944:23552].reshape(out.shape), out)
+
+
+@pytest.mark.parametrize("mutate,message", [
+    (lambda t: t.replace("func.func", "func.fun"), "no func.func"),
+    (lambda t: t.replace("input(%0 :", "input(%99 :", 1), "input operand %99 is not a declared buffer"),
+    (lambda t: t.replace("#VPUIP.nce_task_type<CONV>", "#VPUIP.nce_task_type<CMCONV>"), "CMCONV is not supported"),
+    (lambda t: t.replace("weights(%1 :", "weights_sparsity_map(%1 :", 1), "weights_sparsity_map"),
+    (lambda t: t.replace("outStart = [0, 6, 0]", "outStart = [0, 6]"), "three entries"),
+    (lambda t: t.replace("<CMX_NN> [0] <4608>", "<Register> [0] <4608>"), "section <Register>"),
+    (lambda t: t.replace("PPETask <ADD>", "PPETask <FROBNICATE>"), "unknown PPE mode FROBNICATE"),
+])
+def test_errors_name_the_problem(mutate, message):
+    with pytest.raises(nce.NCEError) as e:
+        vpuip.parse(mutate(TEXT))
+    assert e.value.code == abi.ERROR_INVALID_ARGUMENT and message in e.value.log, e.value.log
+
+
+def test_unbound_sections_and_short_bindings_are_reported():
+    prog = vpuip.parse(TEXT)
+    with pytest.raises(nce.NCEError) as e:
+        prog.task(0)
+    assert "is not bound" in e.value.log
+    prog.bind(vpuip.CMX_NN, 0, np.zeros(16000, np.uint8))
+    with pytest.raises(nce.NCEError) as e:
+        prog.task(1)
+    assert "does not fit" in e.value.log
+
+
+def test_strided_and_aliasless_types():
+    text = TEXT.replace("memref<1x32x12x12x!qMid, #NHWC, [@CMX_NN, 0]>",
+                        "memref<1x32x12x12x!quant.uniform<u8:f32, 5.000000e-02:121>, {order = affine_map<(d0, d1, d2, d3) -> (d0, d2, d3, d1)>, strides = [9216, 1, 768, 64]}, [@CMX_NN, 0]>")
+    prog = vpuip.parse(text)
+    mid = prog.buffer("%3")
+    assert list(mid.strides_bytes) == [9216, 1, 768, 64] and mid.zero_point == 121
+    assert mid.byte_size == 11 * 768 + 11 * 64 + 31 + 1
+
+
+@pytest.mark.gpu
+def test_program_runs_bit_exact(executor):
+    import torch
+    prog = vpuip.parse(TEXT)
+    x, wt, table = _operands(9)
+    cmx = torch.zeros(prog.section_size(vpuip.CMX_NN, 0), dtype=torch.uint8, device="cuda")
+    ddr = torch.zeros(prog.section_size(vpuip.DDR, 0), dtype=torch.uint8, device="cuda")
+    ddr[0:9216] = torch.from_numpy(wt.ravel()).cuda()
+    ddr[9216:9728] = torch.from_numpy(table.view(np.uint8).ravel().copy()).cuda()
+    din = torch.from_numpy(x).cuda()
+    dout = torch.full((1, 12, 12, 32), 0x5A, dtype=torch.uint8, device="cuda")
+    prog.bind(vpuip.CMX_NN, 0, cmx)
+    prog.bind(vpuip.DDR, 0, ddr)
+    prog.bind(vpuip.ARGUMENT, 0, din)
+    prog.bind(vpuip.ARGUMENT, 1, dout)
+    stream = torch.cuda.current_stream().cuda_stream
+    prog.enqueue(executor, stream)
+    executor.synchronize(stream)
+    mid, out = _reference_result(x, wt, table)
+    assert np.array_equal(cmx[14336:18944].cpu().numpy().reshape(mid.shape), mid)
+    assert np.array_equal(dout.cpu().numpy(), out)
