@@ -55,7 +55,9 @@ constexpr FillTable make_fill_table() {
         for (int i = 0; i < 64; ++i) t.b[v][i] = (uint8_t)v;
     return t;
 }
-__device__ const FillTable g_fill = make_fill_table();
+// (not const: a constant-address-space pointer selected against a global one would turn every activation load
+// into a FLAT load, which also counts against the LDS wait counter)
+__device__ FillTable g_fill = make_fill_table();
 
 // Channel (within the slice) that row i of channel fragment f carries: lane (c, q) of the result then
 // holds channels 4*NF*q .. 4*NF*q + 4*NF-1, consecutive, for f = 0..NF-1 and its 4 registers.
