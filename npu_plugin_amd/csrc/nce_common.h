@@ -1,6 +1,7 @@
 // Internal declarations shared by the host side (nce_api.cpp) and the kernel files.
 #pragma once
 
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -82,6 +83,32 @@ __device__ __forceinline__ void store_channels8(uint8_t* p, int64_t sc, uint32_t
         for (int i = 0; i < 8; ++i) p[i * sc] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
     }
 }
+
+// Opt a kernel in to `bytes` of dynamic LDS. The runtime call is made only when a launch needs more than
+// what this kernel was already granted on the current device, so steady-state launches make no runtime
+// call besides the launch itself. One LdsGrant per kernel instantiation (a function-local static).
+struct LdsGrant {
+    static constexpr int kMaxDevices = 64;
+    std::atomic<size_t> granted[kMaxDevices];
+    LdsGrant() {
+        for (auto& g : granted) g.store(0, std::memory_order_relaxed);
+    }
+    hipError_t ensure(const void* kernel, size_t bytes, size_t default_limit) {
+        if (bytes <= default_limit) return hipSuccess;
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < kMaxDevices && granted[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < kMaxDevices) {
+            size_t cur = granted[dev].load(std::memory_order_relaxed);
+            while (cur < bytes && !granted[dev].compare_exchange_weak(cur, bytes, std::memory_order_release)) {
+            }
+        }
+        return hipSuccess;
+    }
+};
 
 hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);
 hipError_t launch_pool(const TaskDev& t, const Box& box, bool is_max, hipStream_t stream);

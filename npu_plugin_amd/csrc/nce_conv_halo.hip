@@ -300,11 +300,8 @@ hipError_t try_launch(ConvArgs a, hipStream_t stream, bool* fits) {
     const unsigned gy = (unsigned)((a.bc + BN - 1) / BN);
     if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
     auto kernel = &conv_halo_kernel<WN, WP, AF, BF, KX>;
-    if (lds > 48 * 1024) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
+    static LdsGrant grant;
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid((unsigned)gx), gy), dim3(NT), lds, stream, a);
     return hipGetLastError();
 }

@@ -34,9 +34,6 @@ struct WresArgs {
     uint32_t ntiles;    // pixel tiles of 16*BF pixels
     uint32_t ngroups;   // workgroups along pixels
     int32_t tpg;        // tiles per workgroup
-    int32_t lu;         // log2 of the units one wave-load covers per weight row
-    int32_t lnblk;      // log2 of the row blocks of a channel slice (64 >> lu rows each)
-    int32_t ui;         // unit passes per row: ceil(nsteps * 4 / 2^lu)
     FastDiv div_icg;    // by IC / 16
     FastDiv div_kx;     // by KX
 };
@@ -80,6 +77,7 @@ __device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
 // and flipped back by an XOR on the packed word.
 struct EpiPack {
     float lo, hi, zp;   // clamp bounds and zero point, including the +128 of signed outputs
+    int32_t ilo, ihi;   // the same bounds as integers: 0 <= ilo <= ihi <= 255
     uint32_t flip;      // 0x80808080 for signed outputs
     double zp_fold;     // folded mode: what B carries on top of the bias term
 };
@@ -87,8 +85,10 @@ struct EpiPack {
 __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     EpiPack e;
     const int32_t sb = pu.lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
-    e.lo = (float)(pu.lo_zp + sb);
-    e.hi = (float)(pu.hi_zp + sb);
+    e.ilo = pu.lo_zp + sb;
+    e.ihi = pu.hi_zp + sb;
+    e.lo = (float)e.ilo;
+    e.hi = (float)e.ihi;
     e.zp = (float)(pu.zp + sb);
     e.flip = sb ? 0x80808080u : 0u;
     e.zp_fold = (double)(pu.zp + sb);
@@ -128,6 +128,11 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
                 if (PMODE == PPE_MODE_INT) {
                     const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
                     wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
+                } else if (PMODE == PPE_MODE_FOLDED) {
+                    // The conversion truncates; below zero that differs from floor, but every value below
+                    // zero (and floor's -1 for a value in (-1, 0)) clamps to ep.ilo >= 0 either way.
+                    const int32_t y = med3_i32((int32_t)__builtin_fma((double)av, M, B), ep.ilo, ep.ihi);
+                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
                 } else {
                     double v = __builtin_floor(__builtin_fma((double)av, M, B));
                     float y;
@@ -159,11 +164,17 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
 
 // D: reduction steps whose activation loads are in flight per wave; the host pads the step count to a
 // multiple of D (the padding steps multiply zero weights by the fill line).
-template <int NF, int BF, int MODE, int D>
+// TRL: transpose the activation operand after loading. The matrix instruction wants lane 16k + p to hold
+// 16-byte piece k of pixel p, which as a load pattern sends the four pieces of a pixel from four
+// different quads of lanes; the texture addresser then works on 64 separate pieces per instruction. When
+// pixels are more than 64 bytes apart that can halve the speed of the whole reduction loop, so there the
+// loads run with lane 4p + k (a pixel's 64 bytes from four neighbouring lanes) and ds_bpermute moves the
+// registers into operand order. With IC == 64 the plain pattern already covers whole lines and is faster.
+template <int NF, int BF, int MODE, int D, bool TRL>
 __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
-    constexpr int WB = 8;      // weight loads in flight per lane while staging
+    constexpr int WB = 4;      // weight loads in flight per lane while staging
     static_assert(NF == 2 || NF == 4, "channel fragments");
     const ConvArgs& a = w.a;
 
@@ -177,8 +188,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps the tile walk in scalar registers
     const int nwaves = blockDim.x >> 6;
-    const int c16 = lane & 15;
-    const int q = lane >> 4;
+    const int c16 = lane & 15;                  // pixel of a fragment this lane holds in matrix layout
+    const int pl = TRL ? lane >> 2 : c16;       // pixel and 16-byte piece this lane loads
+    const int kc = TRL ? lane & 3 : lane >> 4;
+    const int to_mfma = 4 * (4 * c16 + (lane >> 4));  // ds_bpermute source: lane 4p + k feeds lane 16k + p
 
     const int32_t oc0 = a.z0 + blockIdx.y * OCT;
     const int32_t noc = min(OCT, a.z0 + a.bc - oc0);
@@ -186,7 +199,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     if (group >= w.ngroups) return;  // uniform for the whole workgroup
 
     const int axor = (int)a.a_xor;
-    const uint8_t* const fillp = &g_fill.b[(a.fill ^ a.a_xor) & 0xFFu][q * 16];
+    const uint8_t* const fillp = &g_fill.b[(a.fill ^ a.a_xor) & 0xFFu][kc * 16];
     const int S = w.nsteps;
     const uint32_t t_end = min((group + 1) * (uint32_t)w.tpg, w.ntiles);
     uint32_t t = group * (uint32_t)w.tpg + wave;
@@ -203,7 +216,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     auto setup = [&]() {
 #pragma unroll
         for (int x = 0; x < BF; ++x) {
-            const int32_t p = (int32_t)t * BP + 16 * x + c16;
+            const int32_t p = (int32_t)t * BP + 16 * x + pl;
             valid[x] = p < a.M;
             const int32_t pc = valid[x] ? p : a.M - 1;  // lanes past the end compute a duplicate
             const int32_t rr = fdiv(pc, a.div_bw);
@@ -212,8 +225,15 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t by = rr - n * a.bh;
             const int32_t iy0 = (a.y0 + by) * a.SY - a.PT;
             const int32_t ix0 = (a.x0 + bx) * a.SX - a.PL;
-            pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + (MODE == WRES_GENERIC ? 0 : q * 16);
+            pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + (MODE == WRES_GENERIC ? 0 : kc * 16);
             dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0 * a.out_sc;
+            if (TRL) {  // results come out in matrix layout: take the address of pixel c16 from a lane that computed it
+                const uint64_t dl = reinterpret_cast<uint64_t>(dst[x]);
+                const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)dl);
+                const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)(dl >> 32));
+                dst[x] = reinterpret_cast<uint8_t*>(((uint64_t)hi << 32) | lo);
+                valid[x] = (int32_t)t * BP + 16 * x + c16 < a.M;
+            }
             mask0[x] = mask1[x] = 0;
             if (MODE != WRES_FAST) {
                 const uint32_t rows = bit_range(max(0, -iy0), min(a.KY, a.H - iy0));
@@ -234,7 +254,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     // Request the activation operand of the next step for every pixel fragment (raw bytes).
     auto load_b = [&](v4i (&d)[BF]) {
         if (MODE == WRES_GENERIC) {
-            const int u = 4 * ls + q;
+            const int u = 4 * ls + kc;
             const int tap = fdiv(u, w.div_icg);
             const int icg = u - tap * a.ICG;
             const int ky = fdiv(tap, w.div_kx);
@@ -282,17 +302,12 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     }
 
     // ---- stage the channel slice's weights in operand order; per-channel constants ---------------
-    // Lanes split into 64/U rows x U consecutive 16-byte units (U = 2^w.lu covers a row, or is 64), so the
-    // loads of a row are contiguous. A (pass, row block) pair is one such wave-wide load; the first lane
-    // of a row in the last pass also derives the row's PPE constants from its weight-table entry.
+    // The slice is S * NF operand fragments of 1 KiB: (step, channel fragment) -> 16 rows x 64 bytes. A wave
+    // fetches a fragment with lane 4i + k on 16-byte piece k of row i (a row's 64 bytes from four neighbouring
+    // lanes), permutes the registers into operand order (lane 16k + i) and writes the fragment with one
+    // linear, bank-conflict-free store.
     {
-        const int lu = w.lu;
-        const int U = 1 << lu;
-        const int sub = lane & (U - 1);
-        const int rsub = lane >> lu;
-        const int lnblk = w.lnblk;
-        const int k16p = S * 4;
-        const int npairs = w.ui << lnblk;
+        const int li = lane >> 2, lk = lane & 3;
         const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
         // The last wave also derives the per-channel PPE constants (lane = channel) while its weight
         // loads are in flight.
@@ -319,37 +334,47 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 sBc[lane] = B;
             }
         };
-        // (runs at least once: the constants wave may have no weights to stage)
-        for (int m0 = wave, first = 1; first || m0 < npairs; m0 += nwaves * WB, first = 0) {
-            // requests only (nothing here consumes a loaded value) ...
-            uint4 v[WB];
+        // Row (channel) this lane fetches in each channel fragment: the inverse of frag_of_channel.
+        const uint8_t* wrow[NF];
+        bool wrow_ok[NF];
 #pragma unroll
-            for (int j = 0; j < WB; ++j) {
-                const int m = m0 + j * nwaves;
-                const int row = ((m & ((1 << lnblk) - 1)) << (6 - lu)) + rsub;
-                const int u = ((m >> lnblk) << lu) + sub;
-                v[j] = make_uint4(0, 0, 0, 0);
-                if (m < npairs && row < noc && u < w.k16)
-                    v[j] = *reinterpret_cast<const uint4*>(a.w + (int64_t)(oc0 + row) * a.w_soc + (int64_t)u * 16);
+        for (int f = 0; f < NF; ++f) {
+            const int row = 4 * NF * (li >> 2) + 4 * f + (li & 3);
+            wrow_ok[f] = row < noc;
+            wrow[f] = a.w + (int64_t)(oc0 + (wrow_ok[f] ? row : 0)) * a.w_soc + lk * 16;
+        }
+        constexpr int SB = WB / NF;  // steps per batch of loads
+        // (runs at least once: the constants wave may have no weights to stage)
+        for (int s0 = wave, first = 1; first || s0 < S; s0 += nwaves * SB, first = 0) {
+            // requests only (nothing here consumes a loaded value) ...
+            uint4 v[SB][NF];
+#pragma unroll
+            for (int j = 0; j < SB; ++j) {
+                const int st = s0 + j * nwaves;
+                const bool in_k = st < S && 4 * st + lk < w.k16;
+#pragma unroll
+                for (int f = 0; f < NF; ++f) {
+                    // (padding holds the XOR mask itself, so that the unconditional XOR below turns it into zero;
+                    // nothing inside the branch may consume the loaded value, or the loads would serialise)
+                    v[j][f] = make_uint4(a.w_xor, a.w_xor, a.w_xor, a.w_xor);
+                    if (in_k && wrow_ok[f]) v[j][f] = *reinterpret_cast<const uint4*>(wrow[f] + (int64_t)st * 64);
+                }
             }
             if (first && consts_wave) do_consts();  // between the weight requests and their use
-            // ... then the LDS writes
+            // ... then the permutes and LDS writes
 #pragma unroll
-            for (int j = 0; j < WB; ++j) {
-                const int m = m0 + j * nwaves;
-                const int row = ((m & ((1 << lnblk) - 1)) << (6 - lu)) + rsub;
-                const int u = ((m >> lnblk) << lu) + sub;
-                if (m < npairs && u < k16p) {
-                    int f, i;
-                    frag_of_channel<NF>(row, &f, &i);
-                    uint4 x = v[j];
-                    if (row < noc && u < w.k16) {
-                        x.x ^= a.w_xor;
-                        x.y ^= a.w_xor;
-                        x.z ^= a.w_xor;
-                        x.w ^= a.w_xor;
+            for (int j = 0; j < SB; ++j) {
+                const int st = s0 + j * nwaves;
+                if (st < S) {  // uniform
+#pragma unroll
+                    for (int f = 0; f < NF; ++f) {
+                        uint4 x;
+                        x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].x ^ a.w_xor));
+                        x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].y ^ a.w_xor));
+                        x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].z ^ a.w_xor));
+                        x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].w ^ a.w_xor));
+                        *reinterpret_cast<uint4*>(sWt + ((size_t)st * NF + f) * 1024 + lane * 16) = x;
                     }
-                    *reinterpret_cast<uint4*>(sWt + (((u >> 2) * NF + f) * 64 + (u & 3) * 16 + i) * 16) = x;
                 }
             }
         }
@@ -381,9 +406,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         v4i fa[NF];
 #pragma unroll
         for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
-        auto step = [&](v4i (&b)[BF], bool more_a) {
+        auto mma = [&](const v4i (&braw)[BF], bool more_a) {
+            v4i b[BF];
 #pragma unroll
-            for (int x = 0; x < BF; ++x) b[x] = b[x] ^ axor;
+            for (int x = 0; x < BF; ++x) b[x] = braw[x] ^ axor;
 #pragma unroll
             for (int f = 0; f < NF; ++f)
 #pragma unroll
@@ -398,19 +424,49 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
             }
         };
-        for (int g = D; g < S; g += D) {
+        if constexpr (TRL) {
+            // The permute of step s + 1 is issued before the matrix instructions of step s, so its latency
+            // hides behind them; a ring slot is free for its next load once its permute has been issued.
+            auto to_operand = [&](const v4i (&raw)[BF], v4i (&o)[BF]) {
+#pragma unroll
+                for (int x = 0; x < BF; ++x)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[x][r] = __builtin_amdgcn_ds_bpermute(to_mfma, raw[x][r]);
+            };
+            v4i cur[BF], nxt[BF];
+            to_operand(fb[0], cur);
+            for (int g = D; g < S; g += D) {
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    to_operand(fb[(j + 1) % D], nxt);
+                    load_b(fb[j]);
+                    mma(cur, true);
+#pragma unroll
+                    for (int x = 0; x < BF; ++x) cur[x] = nxt[x];
+                }
+            }
 #pragma unroll
             for (int j = 0; j < D; ++j) {
-                step(fb[j], true);
-                load_b(fb[j]);
-            }
-        }
+                if (j + 1 < D) to_operand(fb[j + 1], nxt);
+                mma(cur, j + 1 < D);
 #pragma unroll
-        for (int j = 0; j < D; ++j) step(fb[j], j + 1 < D);
+                for (int x = 0; x < BF; ++x) cur[x] = nxt[x];
+            }
+        } else {
+            for (int g = D; g < S; g += D) {
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    mma(fb[j], true);
+                    load_b(fb[j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < D; ++j) mma(fb[j], j + 1 < D);
+        }
         sum_pass = false;
-        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
-        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sMd, acc, wsum, q, noc, dst, valid, pu, ep);
+        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
+        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
         t += nwaves;
         if (t < t_end) {
             setup();
@@ -421,7 +477,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 
 constexpr size_t kWresLdsCap = 148 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
 
-template <int NF, int BF, int MODE, int D>
+template <int NF, int BF, int MODE, int D, bool TRL>
 hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t stream) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
@@ -433,33 +489,29 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     w.nsteps = (w.nsteps + D - 1) / D * D;
     const size_t lds = (size_t)w.nsteps * NF * 1024;
     if (lds > kWresLdsCap) return hipErrorNotSupported;
-    const int k16p = w.nsteps * 4;
-    w.lu = 2;
-    while (w.lu < 6 && (1 << w.lu) < k16p) ++w.lu;
-    w.lnblk = (NF == 4 ? 6 : 5) - 6 + w.lu;
-    w.ui = (k16p + (1 << w.lu) - 1) >> w.lu;
-    auto kernel = &conv_wres_kernel<NF, BF, MODE, D>;
-    if (lds > 48 * 1024) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
+    auto kernel = &conv_wres_kernel<NF, BF, MODE, D, TRL>;
+    static LdsGrant grant;
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
     return hipGetLastError();
+}
+
+template <int NF, int BF, int D>
+hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
+    // Transposed loads: measured to pay for every kernel larger than 1x1 and for long 1x1 reductions, once
+    // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
+    const bool trl = mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
+    if (mode == WRES_FAST) return trl ? launch_one<NF, BF, WRES_FAST, D, true>(w, nwaves, tpw, stream) : launch_one<NF, BF, WRES_FAST, D, false>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST_MASK) return trl ? launch_one<NF, BF, WRES_FAST_MASK, D, true>(w, nwaves, tpw, stream) : launch_one<NF, BF, WRES_FAST_MASK, D, false>(w, nwaves, tpw, stream);
+    return launch_one<NF, BF, WRES_GENERIC, D, false>(w, nwaves, tpw, stream);
 }
 
 template <int NF, int BF>
 hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
     // Load depth: 4 steps when that needs no padding step (and the ring fits the registers), else 2.
     constexpr int DMAX = BF == 4 ? 2 : 4;
-    if (DMAX == 4 && w.nsteps % 4 == 0) {
-        if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, DMAX>(w, nwaves, tpw, stream);
-        if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, DMAX>(w, nwaves, tpw, stream);
-        return launch_one<NF, BF, WRES_GENERIC, DMAX>(w, nwaves, tpw, stream);
-    }
-    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, 2>(w, nwaves, tpw, stream);
-    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, 2>(w, nwaves, tpw, stream);
-    return launch_one<NF, BF, WRES_GENERIC, 2>(w, nwaves, tpw, stream);
+    if (DMAX == 4 && w.nsteps % 4 == 0) return launch_depth<NF, BF, DMAX>(w, mode, nwaves, tpw, stream);
+    return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
 }
 
 template <int NF>

@@ -255,11 +255,8 @@ hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
     a.zpu = t.in.zp + (t.in.is_signed ? 128 : 0);
     a.fill = (uint32_t)a.zpu * 0x01010101u;
     const size_t lds = MODE == MODE_DW ? (size_t)t.ky * t.kx * SLAB_CH * sizeof(float) : 0;
-    if (lds > 32 * 1024) {  // large depthwise kernels: opt in to more than the default dynamic LDS
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&window_kernel<MODE>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
+    static LdsGrant grant;  // large depthwise kernels: opt in to more than the default dynamic LDS
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE>), lds, 32 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL((window_kernel<MODE>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
     return hipGetLastError();
 }
