@@ -96,8 +96,8 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
 }
 
 template <int NF, int BF, int PMODE>
-__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sMd,
-                                              const v4i (&acc)[NF][BF], const v4i (&wsum)[NF], int q, int noc,
+__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
+                                              const v4i (&acc)[NF][BF], int q, int noc,
                                               uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
                                               const EpiPack& ep) {
     const int ch0 = 4 * NF * q;
@@ -112,15 +112,14 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
             const int c = ch0 + 4 * f + r;
             double M = 0.0, B = 0.0;
             int32_t w2 = 0, bias = 0, corr = 0;
-            // the activation zero point enters as da * (sum of the channel's weights)
+            // (the activation zero point is already in the wave's constants: da * sum of the channel's weights)
             if (PMODE == PPE_MODE_INT) {
                 w2 = s.w2[c];
                 bias = s.bias[c];
-                corr = a.da * wsum[f][r];  // |da| <= 255, |sum w'| < 2^23
+                corr = sCorr[c];
             } else {
                 M = s.M[c];
-                B = __builtin_fma((double)wsum[f][r], sMd[c], s.B[c]);  // exact: 24 x 25 significant bits
-                if (PMODE == PPE_MODE_FOLDED) B += ep.zp_fold;          // floor(x + zp) = floor(x) + zp
+                B = sBfull[c];
             }
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
@@ -176,11 +175,18 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     constexpr int BP = 16 * BF;
     constexpr int WB = 4;      // weight loads in flight per lane while staging
     static_assert(NF == 2 || NF == 4, "channel fragments");
+    static_assert(D >= 2 || !TRL, "the permute of the next step needs a second ring slot");
     const ConvArgs& a = w.a;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
     __shared__ int32_t sW2[OCT], sBias[OCT];
     __shared__ double sM[OCT], sBc[OCT], sMd[OCT];  // scale, bias term, scale * da
+    // Weight sums: every wave leaves the partial sums of the fragments it staged in its row of sWpart; after
+    // the barrier every wave folds the total into its OWN copy of the per-channel constants, so that no
+    // second barrier is needed.
+    __shared__ int32_t sWpart[8][OCT];
+    __shared__ int32_t sCorr[8][OCT];   // integer path: da * sum of weights
+    __shared__ double sBfull[8][OCT];   // FP64 paths: bias term + da * M * sum of weights (+ output zero point)
     __shared__ int32_t sFlags;
     const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
 
@@ -343,6 +349,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             wrow_ok[f] = row < noc;
             wrow[f] = a.w + (int64_t)(oc0 + (wrow_ok[f] ? row : 0)) * a.w_soc + lk * 16;
         }
+        int32_t wpart[NF];  // sum of the (signed) weights this lane staged, per channel fragment
+#pragma unroll
+        for (int f = 0; f < NF; ++f) wpart[f] = 0;
         constexpr int SB = WB / NF;  // steps per batch of loads
         // (runs at least once: the constants wave may have no weights to stage)
         for (int s0 = wave, first = 1; first || s0 < S; s0 += nwaves * SB, first = 0) {
@@ -368,15 +377,28 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 if (st < S) {  // uniform
 #pragma unroll
                     for (int f = 0; f < NF; ++f) {
+                        const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
+                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.x, 0x01010101, wpart[f], false);
+                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.y, 0x01010101, wpart[f], false);
+                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.z, 0x01010101, wpart[f], false);
+                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.w, 0x01010101, wpart[f], false);
                         uint4 x;
-                        x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].x ^ a.w_xor));
-                        x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].y ^ a.w_xor));
-                        x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].z ^ a.w_xor));
-                        x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)(v[j][f].w ^ a.w_xor));
+                        x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.x);
+                        x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.y);
+                        x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.z);
+                        x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.w);
                         *reinterpret_cast<uint4*>(sWt + ((size_t)st * NF + f) * 1024 + lane * 16) = x;
                     }
                 }
             }
+        }
+        // the four lanes of a row add up their pieces; the first of them publishes the wave's partial sum
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+            int32_t p = wpart[f];
+            p += __shfl_xor(p, 1);
+            p += __shfl_xor(p, 2);
+            if (lk == 0) sWpart[wave][4 * NF * (li >> 2) + 4 * f + (li & 3)] = p;
         }
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
@@ -385,15 +407,20 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
     const int pmode = ppe_mode_of(pu, (flags & 1) != 0);
     const EpiPack ep = epi_pack_setup(pu);
+    // This wave's copy of the per-channel constants with the weight sums folded in (lane = channel). The
+    // activation zero point enters as da * (sum of the channel's weights): |da| <= 255, |sum| < 2^23, and
+    // the FP64 product and sum are exact (24 x 25 significant bits).
+    if (lane < OCT) {
+        int32_t ws = 0;
+        for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
+        sCorr[wave][lane] = a.da * ws;
+        double B = __builtin_fma((double)ws, sMd[lane], sBc[lane]);
+        if (pmode == PPE_MODE_FOLDED) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
+        sBfull[wave][lane] = B;
+    }
+    // (same wave writes and reads: program order is enough, the compiler waits on the LDS counter)
 
     // ---- per-wave tile loop -----------------------------------------------------------------------
-    // The per-channel weight sums come out of the matrix unit as well: in its first tile a wave also
-    // multiplies every weight fragment by an all-ones operand (each column of the result is the sum).
-    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-    v4i wsum[NF];
-#pragma unroll
-    for (int f = 0; f < NF; ++f) wsum[f] = v4i{0, 0, 0, 0};
-    bool sum_pass = a.da != 0;
     while (t < t_end) {
         v4i acc[NF][BF];
 #pragma unroll
@@ -414,10 +441,6 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             for (int f = 0; f < NF; ++f)
 #pragma unroll
                 for (int x = 0; x < BF; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], b[x], acc[f][x], 0, 0, 0);
-            if (sum_pass) {
-#pragma unroll
-                for (int f = 0; f < NF; ++f) wsum[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], ones, wsum[f], 0, 0, 0);
-            }
             ap += NF * 1024;
             if (more_a) {
 #pragma unroll
@@ -463,10 +486,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 #pragma unroll
             for (int j = 0; j < D; ++j) mma(fb[j], j + 1 < D);
         }
-        sum_pass = false;
-        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
-        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sMd, acc, wsum, lane >> 4, noc, dst, valid, pu, ep);
+        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
+        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
         t += nwaves;
         if (t < t_end) {
             setup();
@@ -475,7 +497,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     }
 }
 
-constexpr size_t kWresLdsCap = 148 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
+constexpr size_t kWresLdsCap = 144 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
 
 template <int NF, int BF, int MODE, int D, bool TRL>
 hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t stream) {
@@ -500,17 +522,25 @@ template <int NF, int BF, int D>
 hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
     // Transposed loads: measured to pay for every kernel larger than 1x1 and for long 1x1 reductions, once
     // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
-    const bool trl = mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
-    if (mode == WRES_FAST) return trl ? launch_one<NF, BF, WRES_FAST, D, true>(w, nwaves, tpw, stream) : launch_one<NF, BF, WRES_FAST, D, false>(w, nwaves, tpw, stream);
-    if (mode == WRES_FAST_MASK) return trl ? launch_one<NF, BF, WRES_FAST_MASK, D, true>(w, nwaves, tpw, stream) : launch_one<NF, BF, WRES_FAST_MASK, D, false>(w, nwaves, tpw, stream);
+    if constexpr (D >= 2) {
+        const bool trl = mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
+        if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, true>(w, nwaves, tpw, stream);
+        if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, true>(w, nwaves, tpw, stream);
+    }
+    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false>(w, nwaves, tpw, stream);
     return launch_one<NF, BF, WRES_GENERIC, D, false>(w, nwaves, tpw, stream);
 }
 
 template <int NF, int BF>
 hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
-    // Load depth: 4 steps when that needs no padding step (and the ring fits the registers), else 2.
-    constexpr int DMAX = BF == 4 ? 2 : 4;
-    if (DMAX == 4 && w.nsteps % 4 == 0) return launch_depth<NF, BF, DMAX>(w, mode, nwaves, tpw, stream);
+    // Load depth: the deepest of 4, 3, 2 steps that needs no padding step and whose ring fits the registers;
+    // a single-step reduction (1x1 kernel over 64 channels) runs without ring or padding.
+    if (w.nsteps == 1) return launch_depth<NF, BF, 1>(w, mode, nwaves, tpw, stream);
+    if constexpr (BF < 4) {
+        if (w.nsteps % 4 == 0) return launch_depth<NF, BF, 4>(w, mode, nwaves, tpw, stream);
+        if (w.nsteps % 3 == 0) return launch_depth<NF, BF, 3>(w, mode, nwaves, tpw, stream);
+    }
     return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
 }
 
