@@ -34,6 +34,7 @@ struct WresArgs {
     uint32_t ntiles;    // pixel tiles of 16*BF pixels
     uint32_t ngroups;   // workgroups along pixels
     int32_t tpg;        // tiles per workgroup
+    int32_t linear;     // 1x1, stride 1, no padding, whole dense tensors: pixel p sits at p * pixel stride
     FastDiv div_icg;    // by IC / 16
     FastDiv div_kx;     // by KX
 };
@@ -95,6 +96,14 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     return e;
 }
 
+// clamp(y, lo, hi) for lo <= hi as ONE instruction (the compiler cannot prove lo <= hi for run-time bounds and
+// would emit max + min).
+__device__ __forceinline__ int32_t clamp_med3(int32_t y, int32_t lo, int32_t hi) {
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(y), "v"(lo), "v"(hi));
+    return r;
+}
+
 template <int NF, int BF, int PMODE>
 __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
                                               const v4i (&acc)[NF][BF], int q, int noc,
@@ -130,7 +139,7 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
                 } else if (PMODE == PPE_MODE_FOLDED) {
                     // The conversion truncates; below zero that differs from floor, but every value below
                     // zero (and floor's -1 for a value in (-1, 0)) clamps to ep.ilo >= 0 either way.
-                    const int32_t y = med3_i32((int32_t)__builtin_fma((double)av, M, B), ep.ilo, ep.ihi);
+                    const int32_t y = clamp_med3((int32_t)__builtin_fma((double)av, M, B), ep.ilo, ep.ihi);
                     wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
                 } else {
                     double v = __builtin_floor(__builtin_fma((double)av, M, B));
@@ -225,6 +234,14 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t p = (int32_t)t * BP + 16 * x + pl;
             valid[x] = p < a.M;
             const int32_t pc = valid[x] ? p : a.M - 1;  // lanes past the end compute a duplicate
+            if (w.linear) {  // uniform: no decomposition into image, row and column
+                const int32_t ps = (int32_t)t * BP + 16 * x + c16;  // pixel this lane holds in matrix layout
+                pbase[x] = a.in + (int64_t)pc * a.in_sw + (MODE == WRES_GENERIC ? 0 : kc * 16);
+                valid[x] = ps < a.M;
+                dst[x] = a.out + (int64_t)(valid[x] ? ps : a.M - 1) * a.out_sw + oc0 * a.out_sc;
+                mask0[x] = mask1[x] = 1;
+                continue;
+            }
             const int32_t rr = fdiv(pc, a.div_bw);
             const int32_t bx = pc - rr * a.bw;
             const int32_t n = fdiv(rr, a.div_bh);
@@ -476,11 +493,14 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 for (int x = 0; x < BF; ++x) cur[x] = nxt[x];
             }
         } else {
-            for (int g = D; g < S; g += D) {
+            if constexpr (D > 1) {  // (depth 1 is launched for single-step reductions only: the zeroed
+                                    // accumulators then fold into the one matrix instruction's addend)
+                for (int g = D; g < S; g += D) {
 #pragma unroll
-                for (int j = 0; j < D; ++j) {
-                    mma(fb[j], true);
-                    load_b(fb[j]);
+                    for (int j = 0; j < D; ++j) {
+                        mma(fb[j], true);
+                        load_b(fb[j]);
+                    }
                 }
             }
 #pragma unroll
@@ -571,6 +591,9 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     const int64_t ix_lo = (int64_t)a.x0 * a.SX - a.PL, ix_hi = (int64_t)(a.x0 + a.bw - 1) * a.SX - a.PL + a.KX - 1;
     const bool inside = iy_lo >= 0 && iy_hi < a.H && ix_lo >= 0 && ix_hi < a.W;
     const int mode = (a.IC % 64 != 0) ? WRES_GENERIC : (inside ? WRES_FAST : WRES_FAST_MASK);
+    w.linear = a.KY == 1 && a.KX == 1 && a.SY == 1 && a.SX == 1 && a.PT == 0 && a.PL == 0 && a.x0 == 0 && a.y0 == 0 &&
+               a.bw == a.W && a.bh == a.H && a.in_sh == (int64_t)a.W * a.in_sw && a.in_sn == (int64_t)a.H * a.in_sh &&
+               a.out_sh == (int64_t)a.bw * a.out_sw && a.out_sn == (int64_t)a.bh * a.out_sh;
     if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return hipErrorNotSupported;  // one bit per tap, bit 31 stays clear
 
     // Shape of the work: nf channel fragments per slice, bf pixel fragments per wave tile. Measured on
