@@ -3,15 +3,19 @@
 // A workgroup owns one slice of 16*NF output channels and a run of pixel tiles. It stages the WHOLE
 // reduction (KY*KX*IC bytes) of its channels in LDS once, already in MFMA operand order, and after that
 // single barrier its wavefronts never synchronise again: each wave walks its own tiles of 16*BF output
-// pixels, loads the activation operand straight from global memory in the layout the matrix
-// instruction wants, and runs the fused PPE on its accumulators.
+// pixels, loads the activation operand straight from global memory and runs the fused PPE on its
+// accumulators.
 //
 // Why 16x16x64: the B operand of that instruction is 16 pixels x 64 reduction bytes with lane
 // (c = lane % 16, q = lane / 16) holding bytes 16q..16q+15 of pixel c. For NHWC activations those are
-// the four 16-byte quarters of one pixel's 64 consecutive channels, so the 64 lanes of one load cover
-// whole 64-byte runs (a contiguous KiB when IC == 64) instead of 32 half-used lines, and the result
-// layout (lane holds rows 4q..4q+3 of column c) lets the four lanes of a pixel store 64 consecutive
-// output bytes.
+// the four 16-byte quarters of one pixel's 64 consecutive channels, and the result layout (lane holds
+// rows 4q..4q+3 of column c) lets the four lanes of a pixel store 64 consecutive output bytes.
+//
+// Lane order of memory instructions matters more than the bytes they move: a global load whose four
+// neighbouring lanes read one 64-byte run costs the texture addresser a quarter of one whose runs are
+// spread over four quads of lanes, and an LDS store whose lanes share a bank is serialised. Hence the
+// weights (always) and the activations (template flag TRL, when pixels are more than 64 bytes apart) are
+// fetched with lane 4*row + piece and moved into operand order (lane 16*piece + row) with ds_bpermute_b32.
 //
 // The reduction is cut in steps of 64 bytes = four 16-byte units; unit u covers bytes 16u..16u+15 of
 // the OYXI weight row, i.e. tap u / (IC/16), input channels 16 * (u % (IC/16)). With IC a multiple of
