@@ -267,6 +267,9 @@ WRES_SHAPES = [
     (2, 12, 12, 48, 32, (3, 3), (1, 1), (1, 1, 1, 1), 77),     # per-lane tap path: steps straddle taps
     (1, 9, 9, 64, 16, (3, 3), (1, 1), (0, 0, 0, 0), 128),      # 3x3 without padding: every tap inside
     (2, 10, 10, 192, 144, (1, 1), (2, 2), (0, 0, 0, 0), 0),    # 1x1 stride 2, three steps padded to four
+    (1, 12, 12, 128, 48, (3, 3), (1, 1), (0, 0, 0, 0), 128),   # permuted activation loads, every tap inside, ragged channels
+    (2, 9, 9, 192, 64, (3, 3), (1, 1), (1, 1, 1, 1), 99),      # permuted loads with tap masks, 27 steps (depth 3)
+    (1, 5, 7, 2048, 48, (1, 1), (1, 1), (0, 0, 0, 0), 17),     # permuted loads on a long dense 1x1 reduction, partial tile
 ]
 
 
@@ -288,11 +291,20 @@ def test_conv_weights_resident_types_and_modes(executor, monkeypatch, config):
                                                                  round_mode=nce.ROUND_HALF_EVEN)), executor)   # integer PPE path
     check(K.conv_case(424, 2, 14, 14, 64, 64, in_zp=3, scale_lo=20.0, scale_hi=255.0), executor)               # may saturate int32
     check(K.conv_case(425, 2, 14, 14, 64, 64, in_zp=250, ppe=dict(mode=nce.PPE_NOOP, clamp_low=128, clamp_high=255)), executor)
+    # the same with pixels 128 bytes apart and a 3x3 kernel: activation loads in pixel-major lane order
+    wide = dict(k=(3, 3), pads=(1, 1, 1, 1))
+    check(K.conv_case(426, 2, 11, 11, 128, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128, **wide), executor)
+    check(K.conv_case(427, 2, 11, 11, 128, 64, w_signed=False, w_zp=128, in_zp=121, **wide), executor)
+    check(K.conv_case(428, 2, 11, 11, 128, 64, in_zp=3, ppe=dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255,
+                                                                 round_mode=nce.ROUND_HALF_EVEN), **wide), executor)
+    check(K.conv_case(429, 2, 11, 11, 128, 64, in_zp=3, scale_lo=20.0, scale_hi=255.0, **wide), executor)
+    check(K.conv_case(430, 2, 11, 11, 128, 64, in_zp=250, ppe=dict(mode=nce.PPE_NOOP, clamp_low=128, clamp_high=255), **wide), executor)
 
 
 def test_conv_weights_resident_variants(executor, monkeypatch):
     monkeypatch.setenv("NCE_HIP_CONV_WRES", "2,2,4,1")
     test_conv_halo_variants(executor)
+    test_conv_halo_variants(executor, ic=128)   # permuted activation loads, boxes that start inside the image
 
 
 # ---- halo-staged conv kernel: every tile configuration, image-crossing tiles, partial slices -----
@@ -342,13 +354,13 @@ def test_conv_halo_zero_points_and_types(executor, halo_path):
     check(K.conv_case(304, 2, 20, 20, 64, 64, w_signed=False, w_zp=127, in_zp=121), executor)      # falls back to the gather kernel
 
 
-def test_conv_halo_variants(executor):
-    full = K.conv_case(305, 2, 24, 20, 64, 128)
+def test_conv_halo_variants(executor, ic=64):
+    full = K.conv_case(305, 2, 24, 20, ic, 128)
     want = K.run_oracle(full)
-    tiled = K.conv_case(305, 2, 24, 20, 64, 128, variants=[((0, 0, 0), (19, 11, 63)), ((0, 12, 0), (19, 23, 63)),
+    tiled = K.conv_case(305, 2, 24, 20, ic, 128, variants=[((0, 0, 0), (19, 11, 63)), ((0, 12, 0), (19, 23, 63)),
                                                            ((0, 0, 64), (9, 23, 127)), ((10, 0, 64), (19, 23, 127))])
     assert np.array_equal(K.run_hip(tiled, executor), want)
-    part = K.conv_case(305, 2, 24, 20, 64, 128, variants=[((3, 5, 64), (17, 20, 127))])
+    part = K.conv_case(305, 2, 24, 20, ic, 128, variants=[((3, 5, 64), (17, 20, 127))])
     canvas = np.full(part.out_shape, 0x5A, dtype=np.uint8)
     from oracle import nce_oracle
     nce_oracle.run(K.build_task(part, part.input, part.weights, part.table, canvas))
