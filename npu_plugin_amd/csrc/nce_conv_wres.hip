@@ -322,12 +322,6 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 #pragma unroll
         for (int j = 0; j < D; ++j) load_b(fb[j]);
     };
-    // The first tile's activations are requested before anything is waited for.
-    if (t < t_end) {
-        setup();
-        first_loads();
-    }
-
     // ---- stage the channel slice's weights in operand order; per-channel constants ---------------
     // The slice is S * NF operand fragments of 1 KiB: (step, channel fragment) -> 16 rows x 64 bytes. A wave
     // fetches a fragment with lane 4i + k on 16-byte piece k of row i (a row's 64 bytes from four neighbouring
@@ -374,10 +368,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 #pragma unroll
         for (int f = 0; f < NF; ++f) wpart[f] = 0;
         constexpr int SB = WB / NF;  // steps per batch of loads
-        // (runs at least once: the constants wave may have no weights to stage)
-        for (int s0 = wave, first = 1; first || s0 < S; s0 += nwaves * SB, first = 0) {
-            // requests only (nothing here consumes a loaded value) ...
-            uint4 v[SB][NF];
+        uint4 v[SB][NF];
+        // requests only (nothing here consumes a loaded value) ...
+        auto request = [&](int s0) {
 #pragma unroll
             for (int j = 0; j < SB; ++j) {
                 const int st = s0 + j * nwaves;
@@ -390,8 +383,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                     if (in_k && wrow_ok[f]) v[j][f] = *reinterpret_cast<const uint4*>(wrow[f] + (int64_t)st * 64);
                 }
             }
-            if (first && consts_wave) do_consts();  // between the weight requests and their use
-            // ... then the permutes and LDS writes
+        };
+        // ... then the weight sums, permutes and LDS writes
+        auto commit = [&](int s0) {
 #pragma unroll
             for (int j = 0; j < SB; ++j) {
                 const int st = s0 + j * nwaves;
@@ -412,6 +406,19 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                     }
                 }
             }
+        };
+        // The first weights go out before anything else; the pixel bookkeeping of the wave's first tile, its
+        // first activation requests and the constants run while they are in flight.
+        // (No branch around these activation requests - the wait for the weights would otherwise have to cover
+        // them too; a wave without a tile requests the last pixel's data, which setup() clamps to.)
+        request(wave);
+        setup();
+        first_loads();
+        if (consts_wave) do_consts();
+        commit(wave);
+        for (int s0 = wave + nwaves * SB; s0 < S; s0 += nwaves * SB) {
+            request(s0);
+            commit(s0);
         }
         // the four lanes of a row add up their pieces; the first of them publishes the wave's partial sum
 #pragma unroll
