@@ -67,7 +67,11 @@ struct WinArgs {
     int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
 };
 
-template <int MODE>
+// KK = 2, 3: KY == KX == KK known at compile time. All taps of an item are then requested before the first
+// one is used - unconditionally, from coordinates clamped into the image, with out-of-image taps replaced
+// afterwards - so that an item costs one memory round trip instead of one per tap. KK = 0: any window, taps
+// loaded one after the other.
+template <int MODE, int KK>
 __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     // MODE_DW: [tap][SLAB_CH] floats of (w - zp_w); then per-channel FP64 scale constants
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -156,6 +160,31 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         if (MODE == MODE_MAX) {
             // even / odd bytes of each dword as packed u16; order-preserving re-bias for i8
             uint32_t me[4] = {0, 0, 0, 0}, mo[4] = {0, 0, 0, 0};
+            if constexpr (KK > 0) {
+                uint4 v[KK * KK];
+#pragma unroll
+                for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                    for (int kx = 0; kx < KK; ++kx) {
+                        const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
+                        v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                    }
+#pragma unroll
+                for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                    for (int kx = 0; kx < KK; ++kx) {
+                        const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+                        const uint4 va = v[ky * KK + kx];
+                        // (an out-of-image tap becomes 0, the smallest re-biased value: it never wins)
+                        const uint32_t wa[4] = {ok ? va.x ^ a.a_xor : 0u, ok ? va.y ^ a.a_xor : 0u, ok ? va.z ^ a.a_xor : 0u,
+                                                ok ? va.w ^ a.a_xor : 0u};
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            me[d] = pk_max_u16(me[d], wa[d] & 0x00FF00FFu);
+                            mo[d] = pk_max_u16(mo[d], (wa[d] >> 8) & 0x00FF00FFu);
+                        }
+                    }
+            } else
             for (int ky = 0; ky < t.ky; ++ky) {
                 const int32_t iy = iy0 + ky;
                 if ((uint32_t)iy >= (uint32_t)t.in.h) continue;
@@ -189,19 +218,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         float acc[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-        for (int ky = 0; ky < t.ky; ++ky) {
-            const int32_t iy = iy0 + ky;
-            const bool row_in = (uint32_t)iy < (uint32_t)t.in.h;
-            for (int kx = 0; kx < t.kx; ++kx) {
-                const int32_t ix = ix0 + kx;
-                uint4 va = make_uint4(a.fill, a.fill, a.fill, a.fill);
-                if (row_in && (uint32_t)ix < (uint32_t)t.in.w) {
-                    va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
-                    va.x ^= a.a_xor;
-                    va.y ^= a.a_xor;
-                    va.z ^= a.a_xor;
-                    va.w ^= a.a_xor;
-                }
+        auto tap = [&](int ky, int kx, const uint4& va) {
                 const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
                 if (MODE == MODE_DW) {
                     const float4* wp = reinterpret_cast<const float4*>(s_w + (ky * t.kx + kx) * SLAB_CH + (cg << 4));
@@ -216,6 +233,41 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 } else {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[i] += ubyte_f32(wa[i >> 2], i & 3);
+                }
+        };
+        if constexpr (KK > 0) {
+            uint4 v[KK * KK];
+#pragma unroll
+            for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < KK; ++kx) {
+                    const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
+                    v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                }
+#pragma unroll
+            for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < KK; ++kx) {
+                    const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+                    const uint4 r = v[ky * KK + kx];
+                    tap(ky, kx, make_uint4(ok ? r.x ^ a.a_xor : a.fill, ok ? r.y ^ a.a_xor : a.fill, ok ? r.z ^ a.a_xor : a.fill,
+                                           ok ? r.w ^ a.a_xor : a.fill));
+                }
+        } else {
+            for (int ky = 0; ky < t.ky; ++ky) {
+                const int32_t iy = iy0 + ky;
+                const bool row_in = (uint32_t)iy < (uint32_t)t.in.h;
+                for (int kx = 0; kx < t.kx; ++kx) {
+                    const int32_t ix = ix0 + kx;
+                    uint4 va = make_uint4(a.fill, a.fill, a.fill, a.fill);
+                    if (row_in && (uint32_t)ix < (uint32_t)t.in.w) {
+                        va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                        va.x ^= a.a_xor;
+                        va.y ^= a.a_xor;
+                        va.z ^= a.a_xor;
+                        va.w ^= a.a_xor;
+                    }
+                    tap(ky, kx, va);
                 }
             }
         }
@@ -237,8 +289,8 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     }
 }
 
-template <int MODE>
-hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
+template <int MODE, int KK>
+hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
     WinArgs a;
     a.t = t;
     a.box = box;
@@ -256,9 +308,16 @@ hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
     a.fill = (uint32_t)a.zpu * 0x01010101u;
     const size_t lds = MODE == MODE_DW ? (size_t)t.ky * t.kx * SLAB_CH * sizeof(float) : 0;
     static LdsGrant grant;  // large depthwise kernels: opt in to more than the default dynamic LDS
-    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE>), lds, 32 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL((window_kernel<MODE>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE, KK>), lds, 32 * 1024); e != hipSuccess) return e;
+    hipLaunchKernelGGL((window_kernel<MODE, KK>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
     return hipGetLastError();
+}
+
+template <int MODE>
+hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
+    if (t.ky == 3 && t.kx == 3) return launch_window_kk<MODE, 3>(t, box, s);
+    if (t.ky == 2 && t.kx == 2) return launch_window_kk<MODE, 2>(t, box, s);
+    return launch_window_kk<MODE, 0>(t, box, s);
 }
 
 }  // namespace
