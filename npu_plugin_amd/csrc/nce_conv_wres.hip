@@ -64,11 +64,8 @@ __device__ FillTable g_fill = make_fill_table();
 // Channel (within the slice) that row i of channel fragment f carries: lane (c, q) of the result then
 // holds channels 4*NF*q .. 4*NF*q + 4*NF-1, consecutive, for f = 0..NF-1 and its 4 registers.
 template <int NF>
-__device__ __forceinline__ void frag_of_channel(int ch, int* f, int* i) {
-    const int qp = ch / (4 * NF);
-    const int rem = ch - qp * (4 * NF);
-    *f = rem >> 2;
-    *i = 4 * qp + (rem & 3);
+__device__ __forceinline__ int channel_of_frag_row(int f, int i) {
+    return 4 * NF * (i >> 2) + 4 * f + (i & 3);
 }
 
 // bits [lo, hi) of a 32-bit mask (empty when hi <= lo; hi - lo <= 32)
@@ -76,10 +73,10 @@ __device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
     return hi > lo ? ((0xFFFFFFFFu >> (32 - (hi - lo))) << lo) : 0u;
 }
 
-// Wave-uniform constants of the packed FP epilogue: after floor() the value goes to FP32 (exact below
-// 2^24, monotone beyond, and everything beyond is clamped anyway), is clamped with one v_med3_f32 into
-// 0..255 and lands in its output byte with v_cvt_pk_u8_f32. Signed outputs are computed 128 higher
-// and flipped back by an XOR on the packed word.
+// Wave-uniform constants of the FP64 epilogues. Outputs are computed as bytes 0..255: signed outputs 128
+// higher, flipped back by an XOR on the packed word. Folded mode: truncating conversion to int32, one
+// v_med3_i32, byte insert. Slope mode: after floor() the value goes to FP32 (exact below 2^24, monotone
+// beyond, and everything beyond is clamped anyway), one v_med3_f32, v_cvt_pk_u8_f32.
 struct EpiPack {
     float lo, hi, zp;   // clamp bounds and zero point, including the +128 of signed outputs
     int32_t ilo, ihi;   // the same bounds as integers: 0 <= ilo <= ihi <= 255
@@ -174,8 +171,8 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
     }
 }
 
-// D: reduction steps whose activation loads are in flight per wave; the host pads the step count to a
-// multiple of D (the padding steps multiply zero weights by the fill line).
+// D: reduction steps whose activation loads are in flight per wave; the host picks a D that divides the step
+// count where it can and pads the step count otherwise (a padding step multiplies zero weights).
 // TRL: transpose the activation operand after loading. The matrix instruction wants lane 16k + p to hold
 // 16-byte piece k of pixel p, which as a load pattern sends the four pieces of a pixel from four
 // different quads of lanes; the texture addresser then works on 64 separate pieces per instruction. When
@@ -355,12 +352,12 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 sBc[lane] = B;
             }
         };
-        // Row (channel) this lane fetches in each channel fragment: the inverse of frag_of_channel.
+        // Row (channel) this lane fetches in each channel fragment.
         const uint8_t* wrow[NF];
         bool wrow_ok[NF];
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
-            const int row = 4 * NF * (li >> 2) + 4 * f + (li & 3);
+            const int row = channel_of_frag_row<NF>(f, li);
             wrow_ok[f] = row < noc;
             wrow[f] = a.w + (int64_t)(oc0 + (wrow_ok[f] ? row : 0)) * a.w_soc + lk * 16;
         }
@@ -426,7 +423,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             int32_t p = wpart[f];
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
-            if (lk == 0) sWpart[wave][4 * NF * (li >> 2) + 4 * f + (li & 3)] = p;
+            if (lk == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
         }
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
