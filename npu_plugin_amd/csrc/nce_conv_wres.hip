@@ -39,6 +39,7 @@ struct WresArgs {
     uint32_t ngroups;   // workgroups along pixels
     int32_t tpg;        // tiles per workgroup
     int32_t linear;     // 1x1, stride 1, no padding, whole dense tensors: pixel p sits at p * pixel stride
+    int64_t row_adv;    // input offset from the last tap of a kernel row to the first of the next: in_sh - KX * in_sw
     FastDiv div_icg;    // by IC / 16
     FastDiv div_kx;     // by KX
 };
@@ -225,8 +226,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     uint8_t* dst[BF];
     bool valid[BF];
     uint32_t mask0[BF], mask1[BF];  // FAST_MASK: tap bits; GENERIC: row bits, column bits
-    int32_t it_ky = 0, it_kx = 0, it_c64 = 0, it_tap = 0, ls = 0;  // (tap, chunk) the next load belongs to
-    int64_t it_off = 0;
+    int32_t it_kx = 0, it_c64 = 0, it_tap = 0, ls = 0;  // (tap, chunk) the next load belongs to
+    int64_t it_off = 0, tap_off = 0;  // input offset of the next load, of its tap
     v4i fb[D][BF];
 
     auto setup = [&]() {
@@ -272,8 +273,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 }
             }
         }
-        it_ky = it_kx = it_c64 = it_tap = ls = 0;
-        it_off = 0;
+        it_kx = it_c64 = it_tap = ls = 0;
+        it_off = tap_off = 0;
     };
     // Request the activation operand of the next step for every pixel fragment (raw bytes).
     auto load_b = [&](v4i (&d)[BF]) {
@@ -303,11 +304,12 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             if (++it_c64 == w.nc64) {
                 it_c64 = 0;
                 ++it_tap;
+                tap_off += a.in_sw;  // (additions only: the scalar unit has no cheap 64-bit multiply)
                 if (++it_kx == a.KX) {
                     it_kx = 0;
-                    ++it_ky;
+                    tap_off += w.row_adv;
                 }
-                it_off = (int64_t)it_ky * a.in_sh + (int64_t)it_kx * a.in_sw;
+                it_off = tap_off;
                 if (it_tap >= w.ntaps) {  // padding steps: stay on a readable address
                     it_off = 0;
                     it_tap = 31;
@@ -591,6 +593,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     w.ntaps = a.KY * a.KX;
     w.div_icg = make_fastdiv((uint32_t)a.ICG);
     w.div_kx = make_fastdiv((uint32_t)a.KX);
+    w.row_adv = a.in_sh - (int64_t)a.KX * a.in_sw;
     const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
     if (wl2 > kWresLdsCap) return hipErrorNotSupported;
 
