@@ -75,14 +75,13 @@ __device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
 }
 
 // Wave-uniform constants of the FP64 epilogues. Outputs are computed as bytes 0..255: signed outputs 128
-// higher, flipped back by an XOR on the packed word. Folded mode: truncating conversion to int32, one
-// v_med3_i32, byte insert. Slope mode: after floor() the value goes to FP32 (exact below 2^24, monotone
-// beyond, and everything beyond is clamped anyway), one v_med3_f32, v_cvt_pk_u8_f32.
+// higher, flipped back by an XOR on the packed word; truncating conversion to int32, one v_med3_i32, byte
+// insert.
 struct EpiPack {
-    float lo, hi, zp;   // clamp bounds and zero point, including the +128 of signed outputs
-    int32_t ilo, ihi;   // the same bounds as integers: 0 <= ilo <= ihi <= 255
+    int32_t ilo, ihi;   // clamp bounds with the zero point (+128 for signed outputs) added: 0 <= ilo <= ihi <= 255
     uint32_t flip;      // 0x80808080 for signed outputs
-    double zp_fold;     // folded mode: what B carries on top of the bias term
+    double zp_fold;     // what B carries on top of the bias term: the output zero point (+128 for signed outputs)
+    double pcz;         // slope mode: rounding constant of the slope + zp_fold * (1 - slope)
 };
 
 __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
@@ -90,11 +89,9 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     const int32_t sb = pu.lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
     e.ilo = pu.lo_zp + sb;
     e.ihi = pu.hi_zp + sb;
-    e.lo = (float)e.ilo;
-    e.hi = (float)e.ihi;
-    e.zp = (float)(pu.zp + sb);
     e.flip = sb ? 0x80808080u : 0u;
     e.zp_fold = (double)(pu.zp + sb);
+    e.pcz = pu.pc + e.zp_fold - e.zp_fold * pu.pm;  // exact: 8 integer bits, at most 31 fractional bits
     return e;
 }
 
@@ -144,17 +141,14 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
                     const int32_t y = clamp_med3((int32_t)__builtin_fma((double)av, M, B), ep.ilo, ep.ihi);
                     wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
                 } else {
-                    double v = __builtin_floor(__builtin_fma((double)av, M, B));
-                    float y;
-                    if (PMODE == PPE_MODE_SLOPE) {
-                        const double neg = __builtin_floor(__builtin_fma(v, pu.pm, pu.pc));
-                        v = v < 0.0 ? neg : v;
-                        y = (float)v + ep.zp;
-                    } else {
-                        y = (float)v;
-                    }
-                    y = __builtin_amdgcn_fmed3f(y, ep.lo, ep.hi);
-                    wo[x][f] = __builtin_amdgcn_cvt_pk_u8_f32(y, r, wo[x][f]);
+                    // Slope mode, everything shifted up by the output zero point zp (B carries it, as in folded
+                    // mode): tz = t + zp. Below zero the slope applies to floor(t) = floor(tz) - zp, which
+                    // ep.pcz folds in: n = floor(t) * pm + pc + zp, exact. Both candidates are converted by
+                    // truncation - right for values >= 0, and below 0 everything clamps to ep.ilo >= 0.
+                    const double tz = __builtin_fma((double)av, M, B);
+                    const double n = __builtin_fma(__builtin_floor(tz), pu.pm, ep.pcz);
+                    const int32_t y = clamp_med3(tz < ep.zp_fold ? (int32_t)n : (int32_t)tz, ep.ilo, ep.ihi);
+                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
                 }
             }
         }
@@ -442,7 +436,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
         sCorr[wave][lane] = a.da * ws;
         double B = __builtin_fma((double)ws, sMd[lane], sBc[lane]);
-        if (pmode == PPE_MODE_FOLDED) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
+        if (pmode != PPE_MODE_INT) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
         sBfull[wave][lane] = B;
     }
     // (same wave writes and reads: program order is enough, the compiler waits on the LDS counter)
