@@ -39,12 +39,22 @@ struct WresArgs {
     uint32_t ngroups;   // workgroups along pixels
     int32_t tpg;        // tiles per workgroup
     int32_t linear;     // 1x1, stride 1, no padding, whole dense tensors: pixel p sits at p * pixel stride
-    int64_t row_adv;    // input offset from the last tap of a kernel row to the first of the next: in_sh - KX * in_sw
     FastDiv div_icg;    // by IC / 16
     FastDiv div_kx;     // by KX
+    FastDiv div_nc64;   // by nc64
+    int64_t row_adv;    // input offset from the last tap of a kernel row to the first of the next: in_sh - KX * in_sw
 };
 
 enum { WRES_FAST = 0, WRES_FAST_MASK = 1, WRES_GENERIC = 2 };
+
+// Per reduction step (modes 0 and 1): input byte offset of the step's tap and channel chunk relative to the
+// pixel's first tap, and the tap's bit in the per-pixel validity mask (0 for a padding step).
+struct __attribute__((aligned(16))) StepEntry {
+    int32_t off_lo, off_hi;
+    uint32_t tap_bit;
+    int32_t pad;
+};
+constexpr int kMaxSteps = 80;  // 144 KiB / (2 fragments * 1 KiB) = 72 steps, padded to the load depth
 
 // One 64-byte line per byte value: lanes whose tap lies outside the image load the input zero point from
 // here instead of the activation tensor, so every activation load is unconditional (nothing has to
@@ -193,6 +203,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     __shared__ int32_t sCorr[8][OCT];   // integer path: da * sum of weights
     __shared__ double sBfull[8][OCT];   // FP64 paths: bias term + da * M * sum of weights (+ output zero point)
     __shared__ int32_t sFlags;
+    __shared__ StepEntry sStep[kMaxSteps];
     const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
 
     const int tid = threadIdx.x;
@@ -220,8 +231,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     uint8_t* dst[BF];
     bool valid[BF];
     uint32_t mask0[BF], mask1[BF];  // FAST_MASK: tap bits; GENERIC: row bits, column bits
-    int32_t it_kx = 0, it_c64 = 0, it_tap = 0, ls = 0;  // (tap, chunk) the next load belongs to
-    int64_t it_off = 0, tap_off = 0;  // input offset of the next load, of its tap
+    int32_t ls = 0;  // reduction step the next load belongs to
+    // scalar iterator of the kernels that do not read the step table: (tap, chunk) and input offset of the next load
+    int32_t it_kx = 0, it_c64 = 0, it_tap = 0;
+    int64_t it_off = 0, tap_off = 0;
     v4i fb[D][BF];
 
     auto setup = [&]() {
@@ -267,11 +280,29 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 }
             }
         }
-        it_kx = it_c64 = it_tap = ls = 0;
+        ls = 0;
+        it_kx = it_c64 = it_tap = 0;
         it_off = tap_off = 0;
     };
-    // Request the activation operand of the next step for every pixel fragment (raw bytes).
-    auto load_b = [&](v4i (&d)[BF]) {
+    // Entry of reduction step st of the table described at StepEntry.
+    auto step_entry = [&](int st) {
+        const int tap = fdiv(st, w.div_nc64);
+        const int c64 = st - tap * w.nc64;
+        const int ky = fdiv(tap, w.div_kx);
+        const int kx = tap - ky * a.KX;
+        const bool real = tap < w.ntaps;  // padding steps stay on a readable address, their tap bit is clear
+        const int64_t off = real ? (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + c64 * 64 : 0;
+        StepEntry e;
+        e.off_lo = (int32_t)(uint32_t)off;
+        e.off_hi = (int32_t)(off >> 32);
+        e.tap_bit = real ? 1u << tap : 0u;
+        e.pad = 0;
+        return e;
+    };
+    // Request the activation operand of the next step for every pixel fragment (raw bytes). The table of
+    // steps is valid after the workgroup's barrier; the first tile's first requests go out before it and
+    // compute their entries (from_table = false).
+    auto load_b = [&](v4i (&d)[BF], bool from_table = true) {
         if (MODE == WRES_GENERIC) {
             const int u = 4 * ls + kc;
             const int tap = fdiv(u, w.div_icg);
@@ -286,10 +317,11 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 d[x] = *reinterpret_cast<const v4i*>(src);
             }
             ++ls;
-        } else {
+        } else if constexpr (TRL) {
+            // The kernels with permuted loads keep the LDS pipe busy (operand reads, permutes): they walk the
+            // taps with scalar counters instead. Additions only - the scalar unit has no cheap 64-bit multiply.
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
-                // (a padding step re-reads tap 0, whose weights it multiplies are zero; with masks its bit is clear)
                 const uint8_t* src = pbase[x] + it_off;
                 if (MODE == WRES_FAST_MASK) src = ((mask0[x] >> it_tap) & 1u) ? src : fillp;
                 d[x] = *reinterpret_cast<const v4i*>(src);
@@ -298,7 +330,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             if (++it_c64 == w.nc64) {
                 it_c64 = 0;
                 ++it_tap;
-                tap_off += a.in_sw;  // (additions only: the scalar unit has no cheap 64-bit multiply)
+                tap_off += a.in_sw;
                 if (++it_kx == a.KX) {
                     it_kx = 0;
                     tap_off += w.row_adv;
@@ -309,11 +341,23 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                     it_tap = 31;
                 }
             }
+        } else {
+            // Input offset and tap bit of the step come from the table built once per workgroup: one LDS
+            // read instead of a chain of scalar counters, compares and selects per step.
+            const StepEntry e = from_table ? sStep[ls] : step_entry(ls);
+            const int64_t off = ((int64_t)e.off_hi << 32) | (uint32_t)e.off_lo;
+#pragma unroll
+            for (int x = 0; x < BF; ++x) {
+                const uint8_t* src = pbase[x] + off;
+                if (MODE == WRES_FAST_MASK) src = (mask0[x] & e.tap_bit) ? src : fillp;
+                d[x] = *reinterpret_cast<const v4i*>(src);
+            }
+            ++ls;
         }
     };
-    auto first_loads = [&]() {
+    auto first_loads = [&](bool from_table) {
 #pragma unroll
-        for (int j = 0; j < D; ++j) load_b(fb[j]);
+        for (int j = 0; j < D; ++j) load_b(fb[j], from_table);
     };
     // ---- stage the channel slice's weights in operand order; per-channel constants ---------------
     // The slice is S * NF operand fragments of 1 KiB: (step, channel fragment) -> 16 rows x 64 bytes. A wave
@@ -406,7 +450,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         // them too; a wave without a tile requests the last pixel's data, which setup() clamps to.)
         request(wave);
         setup();
-        first_loads();
+        first_loads(false);
         if (consts_wave) do_consts();
         commit(wave);
         for (int s0 = wave + nwaves * SB; s0 < S; s0 += nwaves * SB) {
@@ -421,6 +465,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             p += __shfl_xor(p, 2);
             if (lk == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
         }
+    }
+    if (MODE != WRES_GENERIC && !TRL) {
+        for (int st = tid; st < S; st += (int)blockDim.x) sStep[st] = step_entry(st);
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
 
@@ -516,7 +563,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         t += nwaves;
         if (t < t_end) {
             setup();
-            first_loads();
+            first_loads(true);
         }
     }
 }
@@ -534,7 +581,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     const unsigned gy = (unsigned)((a.bc + OCT - 1) / OCT);
     w.nsteps = (w.nsteps + D - 1) / D * D;
     const size_t lds = (size_t)w.nsteps * NF * 1024;
-    if (lds > kWresLdsCap) return hipErrorNotSupported;
+    if (lds > kWresLdsCap || w.nsteps > kMaxSteps) return hipErrorNotSupported;
     auto kernel = &conv_wres_kernel<NF, BF, MODE, D, TRL>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
@@ -587,6 +634,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     w.ntaps = a.KY * a.KX;
     w.div_icg = make_fastdiv((uint32_t)a.ICG);
     w.div_kx = make_fastdiv((uint32_t)a.KX);
+    w.div_nc64 = make_fastdiv((uint32_t)std::max(1, w.nc64));
     w.row_adv = a.in_sh - (int64_t)a.KX * a.in_sw;
     const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
     if (wl2 > kWresLdsCap) return hipErrorNotSupported;
