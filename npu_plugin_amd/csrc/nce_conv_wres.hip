@@ -184,13 +184,16 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
 // pixels are more than 64 bytes apart that can halve the speed of the whole reduction loop, so there the
 // loads run with lane 4p + k (a pixel's 64 bytes from four neighbouring lanes) and ds_bpermute moves the
 // registers into operand order. With IC == 64 the plain pattern already covers whole lines and is faster.
-template <int NF, int BF, int MODE, int D, bool TRL>
+// TBL: read each step's input offset and tap bit from a table in LDS instead of walking the taps with scalar
+// counters (pays when every step changes tap: kernels larger than 1x1 over 64 input channels).
+template <int NF, int BF, int MODE, int D, bool TRL, bool TBL>
 __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
     constexpr int WB = 4;      // weight loads in flight per lane while staging
     static_assert(NF == 2 || NF == 4, "channel fragments");
     static_assert(D >= 2 || !TRL, "the permute of the next step needs a second ring slot");
+    static_assert(!(TRL && TBL) && !(TBL && MODE == WRES_GENERIC), "the step table serves the plain load order of modes 0 and 1");
     const ConvArgs& a = w.a;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
@@ -317,9 +320,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 d[x] = *reinterpret_cast<const v4i*>(src);
             }
             ++ls;
-        } else if constexpr (TRL) {
-            // The kernels with permuted loads keep the LDS pipe busy (operand reads, permutes): they walk the
-            // taps with scalar counters instead. Additions only - the scalar unit has no cheap 64-bit multiply.
+        } else if constexpr (!TBL) {
+            // Scalar counters walk the taps. Additions only - the scalar unit has no cheap 64-bit multiply.
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
                 const uint8_t* src = pbase[x] + it_off;
@@ -343,7 +345,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             }
         } else {
             // Input offset and tap bit of the step come from the table built once per workgroup: one LDS
-            // read instead of a chain of scalar counters, compares and selects per step.
+            // read instead of a chain of scalar counters, compares and selects per step. (Not for the kernels
+            // with permuted loads, whose LDS pipe is busy with operand reads and permutes, nor for 1x1 kernels,
+            // which never change tap: measured slower there.)
             const StepEntry e = from_table ? sStep[ls] : step_entry(ls);
             const int64_t off = ((int64_t)e.off_hi << 32) | (uint32_t)e.off_lo;
 #pragma unroll
@@ -466,7 +470,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             if (lk == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
         }
     }
-    if (MODE != WRES_GENERIC && !TRL) {
+    if constexpr (TBL) {
         for (int st = tid; st < S; st += (int)blockDim.x) sStep[st] = step_entry(st);
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
@@ -570,7 +574,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 
 constexpr size_t kWresLdsCap = 144 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
 
-template <int NF, int BF, int MODE, int D, bool TRL>
+template <int NF, int BF, int MODE, int D, bool TRL, bool TBL>
 hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t stream) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
@@ -582,7 +586,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     w.nsteps = (w.nsteps + D - 1) / D * D;
     const size_t lds = (size_t)w.nsteps * NF * 1024;
     if (lds > kWresLdsCap || w.nsteps > kMaxSteps) return hipErrorNotSupported;
-    auto kernel = &conv_wres_kernel<NF, BF, MODE, D, TRL>;
+    auto kernel = &conv_wres_kernel<NF, BF, MODE, D, TRL, TBL>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
@@ -595,12 +599,16 @@ hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t 
     // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
     if constexpr (D >= 2) {
         const bool trl = mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
-        if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, true>(w, nwaves, tpw, stream);
-        if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, true>(w, nwaves, tpw, stream);
+        if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, true, false>(w, nwaves, tpw, stream);
+        if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, true, false>(w, nwaves, tpw, stream);
+        // step table: every step changes tap
+        const bool tbl = w.ntaps > 1 && w.nc64 == 1;
+        if (tbl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false, true>(w, nwaves, tpw, stream);
+        if (tbl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false, true>(w, nwaves, tpw, stream);
     }
-    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false>(w, nwaves, tpw, stream);
-    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false>(w, nwaves, tpw, stream);
-    return launch_one<NF, BF, WRES_GENERIC, D, false>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false, false>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false, false>(w, nwaves, tpw, stream);
+    return launch_one<NF, BF, WRES_GENERIC, D, false, false>(w, nwaves, tpw, stream);
 }
 
 template <int NF, int BF>
