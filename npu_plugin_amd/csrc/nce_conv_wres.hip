@@ -399,11 +399,13 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         // Row (channel) this lane fetches in each channel fragment.
         const uint8_t* wrow[NF];
         bool wrow_ok[NF];
+        // (fragment f's row is 4 * f below fragment 0's: one 64-bit multiply, then uniform additions; rows past the
+        // slice's last channel are never dereferenced)
+        const uint8_t* const wrow0 = a.w + (int64_t)(oc0 + channel_of_frag_row<NF>(0, li)) * a.w_soc + lk * 16;
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
-            const int row = channel_of_frag_row<NF>(f, li);
-            wrow_ok[f] = row < noc;
-            wrow[f] = a.w + (int64_t)(oc0 + (wrow_ok[f] ? row : 0)) * a.w_soc + lk * 16;
+            wrow_ok[f] = channel_of_frag_row<NF>(f, li) < noc;
+            wrow[f] = wrow0 + (int64_t)(4 * f) * a.w_soc;
         }
         int32_t wpart[NF];  // sum of the (signed) weights this lane staged, per channel fragment
 #pragma unroll
