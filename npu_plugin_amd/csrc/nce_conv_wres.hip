@@ -105,14 +105,6 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     return e;
 }
 
-// clamp(y, lo, hi) for lo <= hi as ONE instruction (the compiler cannot prove lo <= hi for run-time bounds and
-// would emit max + min).
-__device__ __forceinline__ int32_t clamp_med3(int32_t y, int32_t lo, int32_t hi) {
-    int32_t r;
-    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(y), "v"(lo), "v"(hi));
-    return r;
-}
-
 template <int NF, int BF, int PMODE>
 __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
                                               const v4i (&acc)[NF][BF], int q, int noc,

@@ -23,6 +23,10 @@ struct EltArgs {
     double M, B;  // uniform scale constants (no weight table)
     int32_t c0;   // -(in1_mult * zp_a + in2_mult * zp_b)
     int32_t may_sat;
+    // folded path: outputs are computed as bytes 0..255 (signed outputs 128 higher, flipped back by an XOR on
+    // the packed word; B carries the output zero point and that 128), clamp bounds in that domain
+    int32_t ilo, ihi;
+    uint32_t flip;
 };
 
 // PATH = a PPE_MODE_* value with uniform scale, or PATH_TABLE: integer with a per-channel table.
@@ -68,7 +72,11 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
                 // |acc| < 2^26: 16-bit multipliers times 9-bit values, twice, plus c0
                 const int32_t acc = t.ppe.in1_mult * byte_at<SIGNED>(wa[d], i) + t.ppe.in2_mult * byte_at<SIGNED>(wb[d], i) + a.c0;
                 int32_t y;
-                if (PATH < PPE_MODE_INT) {
+                if (PATH == PPE_MODE_FOLDED) {
+                    // The conversion truncates; below zero that differs from floor, but every value below zero
+                    // clamps to a.ilo >= 0 either way.
+                    y = clamp_med3((int32_t)__builtin_fma((double)acc, a.M, a.B), a.ilo, a.ihi);
+                } else if (PATH < PPE_MODE_INT) {
                     y = ppe_finish_mode<PATH>(__builtin_fma((double)acc, a.M, a.B), pu);
                 } else if (PATH == PPE_MODE_INT) {
                     y = ppe_apply(acc, 0, t.ppe.quant_mult, t.ppe.quant_shift, t.ppe);
@@ -78,7 +86,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
                 }
                 packed = i == 0 ? ((uint32_t)y & 0xFFu) : (packed | (((uint32_t)y & 0xFFu) << (8 * i)));
             }
-            wo[d] = packed;
+            wo[d] = PATH == PPE_MODE_FOLDED ? packed ^ a.flip : packed;
         }
         store_channels16(t.out.data + off_o, FLAT ? 1 : t.out.sc, wo[0], wo[1], wo[2], wo[3]);
     }
@@ -127,7 +135,16 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     if (t.table != nullptr) path = PATH_TABLE;
     else if (shift > kMaxF64Shift || !half_up || a.may_sat || (prelu && prelu_sat)) path = PPE_MODE_INT;
     else path = prelu ? PPE_MODE_SLOPE : PPE_MODE_FOLDED;
-    if (path == PPE_MODE_FOLDED) a.B += (double)t.ppe.zp_out;
+    a.ilo = a.ihi = 0;
+    a.flip = 0;
+    if (path == PPE_MODE_FOLDED) {
+        const int32_t lo_zp = t.ppe.lo + t.ppe.zp_out, hi_zp = t.ppe.hi + t.ppe.zp_out;
+        const int32_t sb = lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
+        a.B += (double)(t.ppe.zp_out + sb);
+        a.ilo = lo_zp + sb;
+        a.ihi = hi_zp + sb;
+        a.flip = sb ? 0x80808080u : 0u;
+    }
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (flat) launch_path<true>(a, path, (int)blocks, stream);

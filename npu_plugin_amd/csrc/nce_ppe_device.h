@@ -108,6 +108,14 @@ __device__ __forceinline__ int32_t med3_i32(int32_t y, int32_t lo, int32_t hi) {
     return min(max(y, lo), hi);
 }
 
+// clamp(y, lo, hi) for lo <= hi as ONE instruction (the compiler cannot prove lo <= hi for run-time bounds and
+// would emit max + min).
+__device__ __forceinline__ int32_t clamp_med3(int32_t y, int32_t lo, int32_t hi) {
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(y), "v"(lo), "v"(hi));
+    return r;
+}
+
 __device__ __forceinline__ double clamp_i32_range(double v) {
     return __builtin_fmin(__builtin_fmax(v, -2147483648.0), 2147483647.0);
 }
