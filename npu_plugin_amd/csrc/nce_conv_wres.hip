@@ -628,6 +628,8 @@ hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStre
 
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     if (a.dw != 0 || a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
+    // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
+    if (a.M > 0x7fffffff - 64 * 1024) return hipErrorNotSupported;
     WresArgs w;
     w.a = a;
     w.k16 = a.KG;
