@@ -235,14 +235,15 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     auto setup = [&]() {
 #pragma unroll
         for (int x = 0; x < BF; ++x) {
-            const int32_t p = (int32_t)t * BP + 16 * x + pl;
-            valid[x] = p < a.M;
-            const int32_t pc = valid[x] ? p : a.M - 1;  // lanes past the end compute a duplicate
+            // (unsigned: a tile index past the end - a wave without a tile - may put the pixel index above 2^31)
+            const uint32_t p = t * BP + 16 * x + pl;
+            valid[x] = p < (uint32_t)a.M;
+            const int32_t pc = valid[x] ? (int32_t)p : a.M - 1;  // lanes past the end compute a duplicate
             if (w.linear) {  // uniform: no decomposition into image, row and column
-                const int32_t ps = (int32_t)t * BP + 16 * x + c16;  // pixel this lane holds in matrix layout
+                const uint32_t ps = t * BP + 16 * x + c16;  // pixel this lane holds in matrix layout
                 pbase[x] = a.in + (int64_t)pc * a.in_sw + (MODE == WRES_GENERIC ? 0 : kc * 16);
-                valid[x] = ps < a.M;
-                dst[x] = a.out + (int64_t)(valid[x] ? ps : a.M - 1) * a.out_sw + oc0 * a.out_sc;
+                valid[x] = ps < (uint32_t)a.M;
+                dst[x] = a.out + (int64_t)(valid[x] ? (int32_t)ps : a.M - 1) * a.out_sw + oc0 * a.out_sc;
                 mask0[x] = mask1[x] = 1;
                 continue;
             }
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
                 const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)dl);
                 const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)(dl >> 32));
                 dst[x] = reinterpret_cast<uint8_t*>(((uint64_t)hi << 32) | lo);
-                valid[x] = (int32_t)t * BP + 16 * x + c16 < a.M;
+                valid[x] = t * BP + 16 * x + c16 < (uint32_t)a.M;
             }
             mask0[x] = mask1[x] = 0;
             if (MODE != WRES_FAST) {
