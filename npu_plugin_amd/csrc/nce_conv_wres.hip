@@ -107,7 +107,7 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
 
 template <int NF, int BF, int PMODE>
 __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
-                                              const v4i (&acc)[NF][BF], int q, int noc,
+                                              const v4i (&acc)[NF][BF], const int32_t (&dws)[BF], int q, int noc,
                                               uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
                                               const EpiPack& ep) {
     const int ch0 = 4 * NF * q;
@@ -133,7 +133,7 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
             }
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
-                const int32_t av = acc[f][x][r];
+                const int32_t av = acc[f][x][r] + dws[x];  // (+ dw * sum of the pixel's activations; 0 when dw == 0)
                 if (PMODE == PPE_MODE_INT) {
                     const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
                     wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
@@ -178,8 +178,17 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
 // registers into operand order. With IC == 64 the plain pattern already covers whole lines and is faster.
 // TBL: read each step's input offset and tap bit from a table in LDS instead of walking the taps with scalar
 // counters (pays when every step changes tap: kernels larger than 1x1 over 64 input channels).
-template <int NF, int BF, int MODE, int D, bool TRL, bool TBL>
+// ASUM: weights whose zero point differs from their storage offset by dw. The product then carries the extra
+// terms dw * (sum of the pixel's activation operand) + K * da * dw: the sum comes out of the matrix unit (one
+// instruction per step and pixel fragment against an all-ones operand, every row of the result is the sum),
+// the constant joins the per-channel constants.
+// LM packs the three flags: 0 plain, 1 TRL, 2 TBL, 3 plain + ASUM, 4 TRL + ASUM.
+enum { LM_PLAIN = 0, LM_TRL = 1, LM_TBL = 2, LM_PLAIN_ASUM = 3, LM_TRL_ASUM = 4 };
+template <int NF, int BF, int MODE, int D, int LM>
 __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
+    constexpr bool TRL = LM == LM_TRL || LM == LM_TRL_ASUM;
+    constexpr bool TBL = LM == LM_TBL;
+    constexpr bool ASUM = LM == LM_PLAIN_ASUM || LM == LM_TRL_ASUM;
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
     constexpr int WB = 4;      // weight loads in flight per lane while staging
@@ -480,8 +489,11 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     if (lane < OCT) {
         int32_t ws = 0;
         for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
-        sCorr[wave][lane] = a.da * ws;
+        // (with a weight zero-point offset dw the constant term S * 64 * da * dw joins; all below 2^30)
+        const int32_t kdd = ASUM ? S * 64 * a.da * a.dw : 0;
+        sCorr[wave][lane] = a.da * ws + kdd;
         double B = __builtin_fma((double)ws, sMd[lane], sBc[lane]);
+        if (ASUM) B = __builtin_fma((double)kdd, sM[lane], B);
         if (pmode != PPE_MODE_INT) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
         sBfull[wave][lane] = B;
     }
@@ -496,6 +508,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             for (int x = 0; x < BF; ++x) acc[f][x] = v4i{0, 0, 0, 0};
         // Steady state: every step consumes one ring slot and refills it for step + D, with no branch
         // around the load, so that the wait before a step covers exactly the loads older than its own.
+        v4i asum[BF];
+#pragma unroll
+        for (int x = 0; x < BF; ++x) asum[x] = v4i{0, 0, 0, 0};
+        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
         const uint8_t* ap = sWt + lane * 16;
         v4i fa[NF];
 #pragma unroll
@@ -508,6 +524,10 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             for (int f = 0; f < NF; ++f)
 #pragma unroll
                 for (int x = 0; x < BF; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], b[x], acc[f][x], 0, 0, 0);
+            if constexpr (ASUM) {
+#pragma unroll
+                for (int x = 0; x < BF; ++x) asum[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b[x], asum[x], 0, 0, 0);
+            }
             ap += NF * 1024;
             if (more_a) {
 #pragma unroll
@@ -556,9 +576,12 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 #pragma unroll
             for (int j = 0; j < D; ++j) mma(fb[j], j + 1 < D);
         }
-        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
-        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, lane >> 4, noc, dst, valid, pu, ep);
+        int32_t dws[BF];  // every row of asum holds the pixel's sum: register 0 of this lane is its column's
+#pragma unroll
+        for (int x = 0; x < BF; ++x) dws[x] = ASUM ? a.dw * asum[x][0] : 0;
+        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
         t += nwaves;
         if (t < t_end) {
             setup();
@@ -569,7 +592,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 
 constexpr size_t kWresLdsCap = 144 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
 
-template <int NF, int BF, int MODE, int D, bool TRL, bool TBL>
+template <int NF, int BF, int MODE, int D, int LM>
 hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t stream) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
@@ -581,7 +604,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     w.nsteps = (w.nsteps + D - 1) / D * D;
     const size_t lds = (size_t)w.nsteps * NF * 1024;
     if (lds > kWresLdsCap || w.nsteps > kMaxSteps) return hipErrorNotSupported;
-    auto kernel = &conv_wres_kernel<NF, BF, MODE, D, TRL, TBL>;
+    auto kernel = &conv_wres_kernel<NF, BF, MODE, D, LM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
@@ -592,22 +615,46 @@ template <int NF, int BF, int D>
 hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
     // Transposed loads: measured to pay for every kernel larger than 1x1 and for long 1x1 reductions, once
     // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
+    const bool trl = D >= 2 && mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
+    if constexpr (D == 2 || D == 4) {
+        if (w.a.dw != 0) {  // activation sums for the weight zero-point term
+            if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
+            if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
+            if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
+            if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
+            return launch_one<NF, BF, WRES_GENERIC, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
+        }
+    }
+    if (w.a.dw != 0) return hipErrorNotSupported;  // (launch_mode sends those tasks to depth 2 or 4)
     if constexpr (D >= 2) {
-        const bool trl = mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
-        if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, true, false>(w, nwaves, tpw, stream);
-        if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, true, false>(w, nwaves, tpw, stream);
+        if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TRL>(w, nwaves, tpw, stream);
+        if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TRL>(w, nwaves, tpw, stream);
         // step table: every step changes tap
         const bool tbl = w.ntaps > 1 && w.nc64 == 1;
-        if (tbl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false, true>(w, nwaves, tpw, stream);
-        if (tbl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false, true>(w, nwaves, tpw, stream);
+        if (tbl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TBL>(w, nwaves, tpw, stream);
+        if (tbl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TBL>(w, nwaves, tpw, stream);
     }
-    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, false, false>(w, nwaves, tpw, stream);
-    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, false, false>(w, nwaves, tpw, stream);
-    return launch_one<NF, BF, WRES_GENERIC, D, false, false>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_PLAIN>(w, nwaves, tpw, stream);
+    if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_PLAIN>(w, nwaves, tpw, stream);
+    return launch_one<NF, BF, WRES_GENERIC, D, LM_PLAIN>(w, nwaves, tpw, stream);
 }
 
 template <int NF, int BF>
 hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
+    if (w.a.dw != 0) {
+        // Depth 4 or 2 only. A padding step must read the fill line (its activations enter the pixel sums), which
+        // the mask mode guarantees: its tap bit is clear.
+        constexpr bool d4 = BF < 4;
+        const bool pad = !(d4 && w.nsteps % 4 == 0) && w.nsteps % 2 != 0;
+        if (pad && mode == WRES_FAST) {
+            if (w.ntaps > 31) return hipErrorNotSupported;
+            mode = WRES_FAST_MASK;
+        }
+        if constexpr (d4) {
+            if (w.nsteps % 4 == 0) return launch_depth<NF, BF, 4>(w, mode, nwaves, tpw, stream);
+        }
+        return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
+    }
     // Load depth: the deepest of 4, 3, 2 steps that needs no padding step and whose ring fits the registers;
     // a single-step reduction (1x1 kernel over 64 channels) runs without ring or padding.
     if (w.nsteps == 1) return launch_depth<NF, BF, 1>(w, mode, nwaves, tpw, stream);
@@ -628,7 +675,7 @@ hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStre
 }  // namespace
 
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
-    if (a.dw != 0 || a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
+    if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
     if (a.M > 0x7fffffff - 64 * 1024) return hipErrorNotSupported;
     WresArgs w;

@@ -301,6 +301,29 @@ def test_conv_weights_resident_types_and_modes(executor, monkeypatch, config):
     check(K.conv_case(430, 2, 11, 11, 128, 64, in_zp=250, ppe=dict(mode=nce.PPE_NOOP, clamp_low=128, clamp_high=255), **wide), executor)
 
 
+WZP_SHAPES = [
+    # (n, h, w, ic, oc, k, s, pads): weights whose zero point is not their storage offset
+    (2, 20, 20, 64, 64, (1, 1), (1, 1), (0, 0, 0, 0)),     # one step, padded to two: the padding step must read the fill line
+    (3, 19, 17, 64, 48, (3, 3), (1, 1), (1, 1, 1, 1)),     # nine steps (padded to ten), tap masks, partial tile
+    (1, 9, 9, 64, 16, (3, 3), (1, 1), (0, 0, 0, 0)),       # no padding of the image, odd step count: mask mode forced
+    (2, 21, 21, 128, 64, (3, 3), (2, 2), (1, 1, 1, 1)),    # permuted loads, 18 steps
+    (1, 12, 12, 256, 48, (3, 3), (1, 1), (0, 0, 0, 0)),    # permuted loads, depth 4, ragged channels
+    (2, 12, 12, 48, 32, (3, 3), (1, 1), (1, 1, 1, 1)),     # per-lane tap path
+    (2, 10, 10, 192, 144, (1, 1), (2, 2), (0, 0, 0, 0)),   # 1x1 stride 2, three steps padded to four
+]
+
+
+@pytest.mark.parametrize("config", ["4,4,8,1", "4,2,8,2", "4,1,4,1", "2,2,4,3", "2,1,8,1"])
+@pytest.mark.parametrize("shape", WZP_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
+def test_conv_weights_resident_weight_zero_point(executor, monkeypatch, shape, config):
+    n, h, w, ic, oc, k, s, pads = shape
+    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    # u8 weights around 117 (offset +11 from the re-biased storage), then i8 weights with zero point 5
+    check(K.conv_case(600 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=131, w_signed=False, w_zp=117, out_zp=9,
+                      ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
+    check(K.conv_case(700 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_signed=True, in_zp=-3, w_signed=True, w_zp=5), executor)
+
+
 def test_conv_weights_resident_variants(executor, monkeypatch):
     monkeypatch.setenv("NCE_HIP_CONV_WRES", "2,2,4,1")
     test_conv_halo_variants(executor)
