@@ -289,9 +289,14 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     // tuning and test knob: 1 = skip the weights-resident kernel, 2 = gather kernel only
     const char* path_env = getenv("NCE_HIP_CONV_PATH");
     const int path = path_env ? atoi(path_env) : 0;
-    hipError_t e = path == 0 ? launch_conv_wres(a, stream) : hipErrorNotSupported;
+    // Reductions too long for one LDS slice: the halo kernel is the faster one for 3-wide kernels (measured on
+    // 3x3 over 1024 channels), the chunked weights-resident kernel for everything else and for what the halo
+    // kernel rejects.
+    hipError_t e = path == 0 ? launch_conv_wres(a, stream, a.KX != 3) : hipErrorNotSupported;
     if (e != hipErrorNotSupported) return e;
     e = path <= 1 ? launch_conv_halo(a, stream) : hipErrorNotSupported;
+    if (e != hipErrorNotSupported) return e;
+    e = path == 0 && a.KX == 3 ? launch_conv_wres(a, stream, true) : hipErrorNotSupported;
     if (e != hipErrorNotSupported) return e;
     return launch_conv_gather(a, stream);
 }

@@ -194,6 +194,7 @@ __device__ __forceinline__ void epi_store(const ConvArgs& a, const EpiSmem& s, v
 hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream);
 // Returns hipErrorNotSupported when the shape does not fit the halo kernel (caller falls back).
 hipError_t launch_conv_halo(const ConvArgs& a, hipStream_t stream);
-hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream);
+// allow_chunked: also take reductions longer than one LDS slice (weights staged chunk by chunk)
+hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked);
 
 }  // namespace nce

@@ -39,6 +39,7 @@ struct WresArgs {
     uint32_t ngroups;   // workgroups along pixels
     int32_t tpg;        // tiles per workgroup
     int32_t linear;     // 1x1, stride 1, no padding, whole dense tensors: pixel p sits at p * pixel stride
+    int32_t cs;         // chunked kernel: reduction steps staged at a time
     FastDiv div_icg;    // by IC / 16
     FastDiv div_kx;     // by KX
     FastDiv div_nc64;   // by nc64
@@ -665,6 +666,317 @@ hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t s
     return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
 }
 
+// ---- reductions longer than LDS: the same kernel shape with the weights staged chunk by chunk ------------
+// For slices whose reduction does not fit LDS (3x3 over 1024 channels, 5x5 over 256, 1x1 over 8192 ...) the
+// workgroup stages CS steps of its weights, synchronises, lets every wave run those steps on its (single) tile,
+// synchronises again and stages the next chunk; accumulators and the activation ring live across chunks.
+// Kept simple: 64-byte-aligned input channels, weights at their storage offset, one tile per wave, load depth 4,
+// permuted activation loads, scalar tap counters, row / column validity bits (any kernel up to 31 x 31).
+template <int NF, int BF>
+__global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
+    constexpr int OCT = 16 * NF;
+    constexpr int BP = 16 * BF;
+    constexpr int D = 4;
+    constexpr int WB = 4;
+    const ConvArgs& a = w.a;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // one chunk: [step][fragment][lane] x 16 bytes
+    __shared__ int32_t sW2[OCT], sBias[OCT];
+    __shared__ double sM[OCT], sBc[OCT], sMd[OCT];
+    __shared__ int32_t sWpart[8][OCT];
+    __shared__ int32_t sCorr[8][OCT];
+    __shared__ double sBfull[8][OCT];
+    __shared__ int32_t sFlags;
+    const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int c16 = lane & 15;
+    const int pl = lane >> 2, kc = lane & 3;          // pixel and 16-byte piece this lane loads
+    const int to_mfma = 4 * (4 * c16 + (lane >> 4));  // ds_bpermute source: lane 4p + k feeds lane 16k + p
+
+    const int32_t oc0 = a.z0 + blockIdx.y * OCT;
+    const int32_t noc = min(OCT, a.z0 + a.bc - oc0);
+    const uint32_t group = xcd_tile(blockIdx.x, w.ngroups);
+    if (group >= w.ngroups) return;  // uniform for the whole workgroup
+
+    const int axor = (int)a.a_xor;
+    const uint8_t* const fillp = &g_fill.b[(a.fill ^ a.a_xor) & 0xFFu][kc * 16];
+    const int S = w.nsteps;   // padded to a multiple of D
+    const int CS = w.cs;      // steps per chunk, a multiple of D
+    const uint32_t t = group * (uint32_t)w.tpg + wave;  // this wave's tile (one per wave)
+    const bool has_tile = t < w.ntiles;
+
+    // ---- the tile: pixel addresses and validity bits (a wave without a tile works on the last pixel, stores nothing)
+    const uint8_t* pbase[BF];
+    uint8_t* dst[BF];
+    bool valid[BF];
+    uint32_t rows[BF], cols[BF];
+#pragma unroll
+    for (int x = 0; x < BF; ++x) {
+        const uint32_t p = t * BP + 16 * x + pl;
+        const bool in_range = p < (uint32_t)a.M;
+        const int32_t pc = in_range ? (int32_t)p : a.M - 1;
+        const int32_t rr = fdiv(pc, a.div_bw);
+        const int32_t bx = pc - rr * a.bw;
+        const int32_t n = fdiv(rr, a.div_bh);
+        const int32_t by = rr - n * a.bh;
+        const int32_t iy0 = (a.y0 + by) * a.SY - a.PT;
+        const int32_t ix0 = (a.x0 + bx) * a.SX - a.PL;
+        pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + kc * 16;
+        uint8_t* d = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0 * a.out_sc;
+        // results come out in matrix layout: take the address of pixel c16 from a lane that computed it
+        const uint64_t dl = reinterpret_cast<uint64_t>(d);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)dl);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)(dl >> 32));
+        dst[x] = reinterpret_cast<uint8_t*>(((uint64_t)hi << 32) | lo);
+        valid[x] = has_tile && t * BP + 16 * x + c16 < (uint32_t)a.M;
+        rows[x] = bit_range(max(0, -iy0), min(a.KY, a.H - iy0));  // bit 31 stays clear (KY, KX <= 31): padding steps
+        cols[x] = bit_range(max(0, -ix0), min(a.KX, a.W - ix0));
+    }
+    // scalar walk over (kernel row, kernel column, 64-byte channel chunk); additions only
+    int32_t it_ky = 0, it_kx = 0, it_c64 = 0;
+    int64_t it_off = 0, tap_off = 0;
+    v4i fb[D][BF];
+    auto load_b = [&](v4i (&d)[BF]) {
+#pragma unroll
+        for (int x = 0; x < BF; ++x) {
+            const uint8_t* src = pbase[x] + it_off;
+            src = ((rows[x] >> it_ky) & (cols[x] >> it_kx) & 1u) ? src : fillp;
+            d[x] = *reinterpret_cast<const v4i*>(src);
+        }
+        it_off += 64;
+        if (++it_c64 == w.nc64) {
+            it_c64 = 0;
+            tap_off += a.in_sw;
+            if (++it_kx == a.KX) {
+                it_kx = 0;
+                tap_off += w.row_adv;
+                if (++it_ky >= a.KY) {  // padding steps: a readable address, a clear validity bit
+                    it_ky = 31;
+                    tap_off = 0;
+                }
+            }
+            it_off = tap_off;
+        }
+    };
+
+    // ---- weight staging (see conv_wres_kernel) ---------------------------------------------------------------
+    const int li = lane >> 2, lk = lane & 3;
+    const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
+    const bool consts_wave = wave == nwaves - 1;
+    int32_t tw2 = 0, tbias = 0;
+    if (consts_wave && lane < noc) {
+        const int32_t* trow = a.table + (int64_t)(oc0 + lane) * a.table_stride;
+        tw2 = trow[2];
+        tbias = trow[3];
+    }
+    const uint8_t* wrow[NF];
+    bool wrow_ok[NF];
+    const uint8_t* const wrow0 = a.w + (int64_t)(oc0 + channel_of_frag_row<NF>(0, li)) * a.w_soc + lk * 16;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+        wrow_ok[f] = channel_of_frag_row<NF>(f, li) < noc;
+        wrow[f] = wrow0 + (int64_t)(4 * f) * a.w_soc;
+    }
+    int32_t wpart[NF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) wpart[f] = 0;
+    constexpr int SB = WB / NF;
+    uint4 v[SB][NF];
+    auto request = [&](int s0, int send) {
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            const int st = s0 + j * nwaves;
+            const bool in_k = st < send && 4 * st + lk < w.k16;
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                v[j][f] = make_uint4(a.w_xor, a.w_xor, a.w_xor, a.w_xor);  // (becomes zero under the XOR below)
+                if (in_k && wrow_ok[f]) v[j][f] = *reinterpret_cast<const uint4*>(wrow[f] + (int64_t)st * 64);
+            }
+        }
+    };
+    auto commit = [&](int s0, int sbase, int send) {
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            const int st = s0 + j * nwaves;
+            if (st < send) {  // uniform
+#pragma unroll
+                for (int f = 0; f < NF; ++f) {
+                    const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
+                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.x, 0x01010101, wpart[f], false);
+                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.y, 0x01010101, wpart[f], false);
+                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.z, 0x01010101, wpart[f], false);
+                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.w, 0x01010101, wpart[f], false);
+                    uint4 x;
+                    x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.x);
+                    x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.y);
+                    x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.z);
+                    x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.w);
+                    *reinterpret_cast<uint4*>(sWt + ((size_t)(st - sbase) * NF + f) * 1024 + lane * 16) = x;
+                }
+            }
+        }
+    };
+    auto stage_chunk = [&](int sbase, int send) {
+        for (int s0 = sbase + wave; s0 < send; s0 += nwaves * SB) {
+            request(s0, send);
+            commit(s0, sbase, send);
+        }
+    };
+
+    // first chunk: the activation requests of the first D steps go out while its first weights are in flight
+    const int send0 = min(CS, S);
+    request(wave, send0);
+#pragma unroll
+    for (int j = 0; j < D; ++j) load_b(fb[j]);
+    if (consts_wave) {
+        const int32_t mult = table_mult(tw2), shift = table_shift(tw2);
+        const bool bad = lane < OCT && shift > kMaxF64Shift;
+        const bool sat = lane < OCT && ppe_may_saturate(acc_bound, tbias, mult, shift);
+        const int wf = (__any(bad) ? 1 : 0) | (__any(sat) ? 2 : 0);
+        if (lane == 0) sFlags = wf;
+        if (lane < OCT) {
+            const double M = ppe_scale_M(mult, shift);
+            sW2[lane] = tw2;
+            sBias[lane] = tbias;
+            sM[lane] = M;
+            sMd[lane] = M * (double)a.da;
+            sBc[lane] = ppe_scale_B(tbias, M, shift, a.ppe.round_mode);
+        }
+    }
+    commit(wave, 0, send0);
+    for (int s0 = wave + nwaves * SB; s0 < send0; s0 += nwaves * SB) {
+        request(s0, send0);
+        commit(s0, 0, send0);
+    }
+
+    // ---- chunks ------------------------------------------------------------------------------------------------
+    v4i acc[NF][BF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int x = 0; x < BF; ++x) acc[f][x] = v4i{0, 0, 0, 0};
+    auto to_operand = [&](const v4i (&raw)[BF], v4i (&o)[BF]) {
+#pragma unroll
+        for (int x = 0; x < BF; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[x][r] = __builtin_amdgcn_ds_bpermute(to_mfma, raw[x][r]);
+    };
+    v4i cur[BF], nxt[BF];
+    to_operand(fb[0], cur);
+    for (int sbase = 0; sbase < S; sbase += CS) {
+        const int send = min(sbase + CS, S);
+        if (sbase > 0) stage_chunk(sbase, send);
+        if (send == S) {  // every weight has passed through: publish the wave's partial sums
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                int32_t p = wpart[f];
+                p += __shfl_xor(p, 1);
+                p += __shfl_xor(p, 2);
+                if (lk == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
+            }
+        }
+        __syncthreads();  // the chunk is in LDS
+        const uint8_t* ap = sWt + lane * 16;
+        v4i fa[NF];
+#pragma unroll
+        for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
+        auto mma = [&](bool more_a) {
+            v4i b[BF];
+#pragma unroll
+            for (int x = 0; x < BF; ++x) b[x] = cur[x] ^ axor;
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+#pragma unroll
+                for (int x = 0; x < BF; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], b[x], acc[f][x], 0, 0, 0);
+            ap += NF * 1024;
+            if (more_a) {
+#pragma unroll
+                for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
+            }
+        };
+        for (int g = sbase; g < send; g += D) {
+            const bool last_in_chunk = g + D >= send;
+            if (g + D < S) {  // uniform: steps remain after this group, its ring slots are refilled
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    to_operand(fb[(j + 1) % D], nxt);
+                    load_b(fb[j]);
+                    mma(!(last_in_chunk && j == D - 1));
+#pragma unroll
+                    for (int x = 0; x < BF; ++x) cur[x] = nxt[x];
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    if (j + 1 < D) to_operand(fb[j + 1], nxt);
+                    mma(j + 1 < D);
+#pragma unroll
+                    for (int x = 0; x < BF; ++x) cur[x] = nxt[x];
+                }
+            }
+        }
+        if (send < S) __syncthreads();  // every wave is done with the chunk before it is overwritten
+    }
+
+    const int flags = sFlags;
+    const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
+    const int pmode = ppe_mode_of(pu, (flags & 1) != 0);
+    const EpiPack ep = epi_pack_setup(pu);
+    if (lane < OCT) {
+        int32_t ws = 0;
+        for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
+        sCorr[wave][lane] = a.da * ws;
+        double B = __builtin_fma((double)ws, sMd[lane], sBc[lane]);
+        if (pmode != PPE_MODE_INT) B += ep.zp_fold;
+        sBfull[wave][lane] = B;
+    }
+    const int32_t dws[BF] = {};
+    if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+    else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+    else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+}
+
+template <int NF, int BF>
+hipError_t launch_chunked(WresArgs& w, int nwaves, hipStream_t stream) {
+    constexpr int OCT = 16 * NF;
+    constexpr int BP = 16 * BF;
+    const ConvArgs& a = w.a;
+    w.ntiles = (uint32_t)(((int64_t)a.M + BP - 1) / BP);
+    w.tpg = nwaves;  // one tile per wave
+    w.ngroups = (w.ntiles + w.tpg - 1) / w.tpg;
+    const unsigned gy = (unsigned)((a.bc + OCT - 1) / OCT);
+    w.nsteps = (w.nsteps + 3) / 4 * 4;
+    w.cs = (int32_t)(kWresLdsCap / ((size_t)NF * 1024)) / 4 * 4;
+    const size_t lds = (size_t)std::min(w.cs, w.nsteps) * NF * 1024;
+    auto kernel = &conv_wres_chunked_kernel<NF, BF>;
+    static LdsGrant grant;
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
+    return hipGetLastError();
+}
+
+// Long reductions: 32 channels x 72 steps per chunk; the pixel tile as large as still gives ~1500 wave tiles.
+hipError_t launch_conv_wres_chunked(WresArgs& w, hipStream_t stream) {
+    const ConvArgs& a = w.a;
+    if (a.IC % 64 != 0 || a.dw != 0 || a.KY > 31 || a.KX > 31) return hipErrorNotSupported;
+    const int64_t slices = (a.bc + 31) / 32;
+    int bf = (((int64_t)a.M + 31) / 32) * slices >= 1500 ? 2 : 1;
+    int nw = 8;
+    if (const char* forced = getenv("NCE_HIP_CONV_WRES")) {  // "nf,bf,nwaves,tiles_per_wave": bf (1, 2) and nwaves apply
+        int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
+        if (sscanf(forced, "%d,%d,%d,%d", &fnf, &fbf, &fnw, &ftpw) == 4) {
+            if (fbf == 1 || fbf == 2) bf = fbf;
+            if (fnw >= 1 && fnw <= 8) nw = fnw;
+        }
+    }
+    if (bf == 2) return launch_chunked<2, 2>(w, nw, stream);
+    return launch_chunked<2, 1>(w, nw, stream);
+}
+
 template <int NF>
 hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream) {
     if (bf == 4) return launch_mode<NF, 4>(w, mode, nwaves, tpw, stream);
@@ -674,7 +986,7 @@ hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStre
 
 }  // namespace
 
-hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
+hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked) {
     if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
     if (a.M > 0x7fffffff - 64 * 1024) return hipErrorNotSupported;
@@ -689,7 +1001,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream) {
     w.div_nc64 = make_fastdiv((uint32_t)std::max(1, w.nc64));
     w.row_adv = a.in_sh - (int64_t)a.KX * a.in_sw;
     const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
-    if (wl2 > kWresLdsCap) return hipErrorNotSupported;
+    if (wl2 > kWresLdsCap) return allow_chunked ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
 
     // every tap of every output pixel of the box inside the image?
     const int64_t iy_lo = (int64_t)a.y0 * a.SY - a.PT, iy_hi = (int64_t)(a.y0 + a.bh - 1) * a.SY - a.PT + a.KY - 1;

@@ -458,3 +458,24 @@ def test_odu_permutation_variants_leave_other_bytes_alone(executor):
     case = K.conv_case(607, 1, 12, 12, 64, 64, variants=[((2, 3, 16), (9, 10, 47))])
     got, want = _permuted_run(case, "nchw", executor)
     assert np.array_equal(got, want) and (want == 0x5A).sum() > want.size // 2
+
+
+# ---- reductions longer than one LDS slice: weights staged chunk by chunk ------------------------------
+
+LONG_K_SHAPES = [
+    # (n, h, w, ic, oc, k, s, pads)
+    (1, 6, 6, 1024, 48, (3, 3), (1, 1), (1, 1, 1, 1)),     # 9216 bytes: two chunks, tap masks, ragged channels
+    (2, 7, 5, 256, 32, (5, 5), (1, 1), (2, 2, 2, 2)),      # 6400 bytes, 25 taps
+    (1, 9, 9, 128, 64, (7, 7), (2, 2), (3, 3, 3, 3)),      # 49 taps (more than the tap-mask kernels take), stride 2
+    (1, 5, 7, 8192, 32, (1, 1), (1, 1), (0, 0, 0, 0)),     # 1x1 over 8192 channels: two chunks, partial tile
+    (1, 4, 4, 4672, 32, (1, 1), (1, 1), (0, 0, 0, 0)),     # 73 steps: padded to 76, second chunk of four steps
+]
+
+
+@pytest.mark.parametrize("config", ["2,1,8,1", "2,2,4,1", "2,1,3,1"])
+@pytest.mark.parametrize("shape", LONG_K_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
+def test_conv_long_reduction(executor, monkeypatch, shape, config):
+    n, h, w, ic, oc, k, s, pads = shape
+    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    check(K.conv_case(800 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=119, out_zp=3,
+                      ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
