@@ -670,9 +670,9 @@ hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t s
 // For slices whose reduction does not fit LDS (3x3 over 1024 channels, 5x5 over 256, 1x1 over 8192 ...) the
 // workgroup stages CS steps of its weights, synchronises, lets every wave run those steps on its (single) tile,
 // synchronises again and stages the next chunk; accumulators and the activation ring live across chunks.
-// Kept simple: 64-byte-aligned input channels, weights at their storage offset, one tile per wave, load depth 4,
-// permuted activation loads, scalar tap counters, row / column validity bits (any kernel up to 31 x 31).
-template <int NF, int BF>
+// Kept simple: 64-byte-aligned input channels, one tile per wave, load depth 4, permuted activation loads, scalar
+// tap counters, row / column validity bits (any kernel up to 31 x 31). ASUM as in conv_wres_kernel.
+template <int NF, int BF, bool ASUM>
 __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
@@ -867,6 +867,10 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
     };
     v4i cur[BF], nxt[BF];
     to_operand(fb[0], cur);
+    v4i asum[BF];
+#pragma unroll
+    for (int x = 0; x < BF; ++x) asum[x] = v4i{0, 0, 0, 0};
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
     for (int sbase = 0; sbase < S; sbase += CS) {
         const int send = min(sbase + CS, S);
         if (sbase > 0) stage_chunk(sbase, send);
@@ -892,6 +896,10 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
             for (int f = 0; f < NF; ++f)
 #pragma unroll
                 for (int x = 0; x < BF; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], b[x], acc[f][x], 0, 0, 0);
+            if constexpr (ASUM) {
+#pragma unroll
+                for (int x = 0; x < BF; ++x) asum[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b[x], asum[x], 0, 0, 0);
+            }
             ap += NF * 1024;
             if (more_a) {
 #pragma unroll
@@ -929,18 +937,23 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
     if (lane < OCT) {
         int32_t ws = 0;
         for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
-        sCorr[wave][lane] = a.da * ws;
+        // (the host rejects reductions for which S * 64 * da * dw or dw * a pixel's sum could leave int32)
+        const int32_t kdd = ASUM ? S * 64 * a.da * a.dw : 0;
+        sCorr[wave][lane] = a.da * ws + kdd;
         double B = __builtin_fma((double)ws, sMd[lane], sBc[lane]);
+        if (ASUM) B = __builtin_fma((double)kdd, sM[lane], B);
         if (pmode != PPE_MODE_INT) B += ep.zp_fold;
         sBfull[wave][lane] = B;
     }
-    const int32_t dws[BF] = {};
+    int32_t dws[BF];
+#pragma unroll
+    for (int x = 0; x < BF; ++x) dws[x] = ASUM ? a.dw * asum[x][0] : 0;
     if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
     else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
     else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
 }
 
-template <int NF, int BF>
+template <int NF, int BF, bool ASUM>
 hipError_t launch_chunked(WresArgs& w, int nwaves, hipStream_t stream) {
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
@@ -952,7 +965,7 @@ hipError_t launch_chunked(WresArgs& w, int nwaves, hipStream_t stream) {
     w.nsteps = (w.nsteps + 3) / 4 * 4;
     w.cs = (int32_t)(kWresLdsCap / ((size_t)NF * 1024)) / 4 * 4;
     const size_t lds = (size_t)std::min(w.cs, w.nsteps) * NF * 1024;
-    auto kernel = &conv_wres_chunked_kernel<NF, BF>;
+    auto kernel = &conv_wres_chunked_kernel<NF, BF, ASUM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
@@ -962,7 +975,9 @@ hipError_t launch_chunked(WresArgs& w, int nwaves, hipStream_t stream) {
 // Long reductions: 32 channels x 72 steps per chunk; the pixel tile as large as still gives ~1500 wave tiles.
 hipError_t launch_conv_wres_chunked(WresArgs& w, hipStream_t stream) {
     const ConvArgs& a = w.a;
-    if (a.IC % 64 != 0 || a.dw != 0 || a.KY > 31 || a.KX > 31) return hipErrorNotSupported;
+    if (a.IC % 64 != 0 || a.KY > 31 || a.KX > 31) return hipErrorNotSupported;
+    // (weight zero-point offset: keep S * 64 * da * dw and dw * pixel sums inside int32 for the integer PPE path)
+    if (a.dw != 0 && (int64_t)(w.nsteps + 3) * 64 * 255 * 255 > 0x7fffffffLL) return hipErrorNotSupported;
     const int64_t slices = (a.bc + 31) / 32;
     int bf = (((int64_t)a.M + 31) / 32) * slices >= 1500 ? 2 : 1;
     int nw = 8;
@@ -973,8 +988,8 @@ hipError_t launch_conv_wres_chunked(WresArgs& w, hipStream_t stream) {
             if (fnw >= 1 && fnw <= 8) nw = fnw;
         }
     }
-    if (bf == 2) return launch_chunked<2, 2>(w, nw, stream);
-    return launch_chunked<2, 1>(w, nw, stream);
+    if (a.dw != 0) return bf == 2 ? launch_chunked<2, 2, true>(w, nw, stream) : launch_chunked<2, 1, true>(w, nw, stream);
+    return bf == 2 ? launch_chunked<2, 2, false>(w, nw, stream) : launch_chunked<2, 1, false>(w, nw, stream);
 }
 
 template <int NF>
@@ -1011,7 +1026,8 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     w.linear = a.KY == 1 && a.KX == 1 && a.SY == 1 && a.SX == 1 && a.PT == 0 && a.PL == 0 && a.x0 == 0 && a.y0 == 0 &&
                a.bw == a.W && a.bh == a.H && a.in_sh == (int64_t)a.W * a.in_sw && a.in_sn == (int64_t)a.H * a.in_sh &&
                a.out_sh == (int64_t)a.bw * a.out_sw && a.out_sn == (int64_t)a.bh * a.out_sh;
-    if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return hipErrorNotSupported;  // one bit per tap, bit 31 stays clear
+    // one bit per tap, bit 31 stays clear; larger kernels take the chunked kernel's row / column bits
+    if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return allow_chunked ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
 
     // Shape of the work: nf channel fragments per slice, bf pixel fragments per wave tile. Measured on
     // MI355X over the ResNet-50 layer shapes, the best shape is always the LARGEST tile that still

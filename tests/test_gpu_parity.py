@@ -479,3 +479,11 @@ def test_conv_long_reduction(executor, monkeypatch, shape, config):
     monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
     check(K.conv_case(800 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=119, out_zp=3,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
+    # weights whose zero point is not their storage offset
+    check(K.conv_case(900 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=119, w_signed=False, w_zp=140), executor)
+
+
+def test_conv_wide_padded_kernel_on_chunked_kernel(executor):
+    # 7x7 with padding over 64 channels fits LDS but needs more than 31 tap bits: row / column bits of the chunked kernel
+    check(K.conv_case(512, 2, 13, 11, 64, 48, k=(7, 7), s=(1, 1), pads=(3, 3, 3, 3), in_zp=100), executor)
+    check(K.conv_case(513, 1, 13, 11, 128, 32, k=(6, 6), s=(2, 2), pads=(2, 2, 3, 3), in_zp=7, w_signed=False, w_zp=131), executor)
