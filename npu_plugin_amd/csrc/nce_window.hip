@@ -67,7 +67,7 @@ struct WinArgs {
     int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
 };
 
-// KK = 2, 3: KY == KX == KK known at compile time. All taps of an item are then requested before the first
+// KK = 2, 3, 5: KY == KX == KK known at compile time. All taps of an item are then requested before the first
 // one is used - unconditionally, from coordinates clamped into the image, with out-of-image taps replaced
 // afterwards - so that an item costs one memory round trip instead of one per tap. KK = 0: any window, taps
 // loaded one after the other.
@@ -317,6 +317,7 @@ template <int MODE>
 hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
     if (t.ky == 3 && t.kx == 3) return launch_window_kk<MODE, 3>(t, box, s);
     if (t.ky == 2 && t.kx == 2) return launch_window_kk<MODE, 2>(t, box, s);
+    if (t.ky == 5 && t.kx == 5) return launch_window_kk<MODE, 5>(t, box, s);
     return launch_window_kk<MODE, 0>(t, box, s);
 }
 
