@@ -87,56 +87,48 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     float* s_w = reinterpret_cast<float*>(smem);
 
     // ---- per-channel constants ---------------------------------------------------------------
-    // pass 1: which PPE specialisation the block runs (uniform); pass 2: the constants for it
-    int bad_shift = 0, small_shift = 0;
-    if (MODE != MODE_MAX) {
-        for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
-            int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
-            if (t.table != nullptr) {
-                const int32_t* row = t.table + (int64_t)(box.z0 + slab0 * 16 + ch) * t.table_stride;
-                mult = table_mult(row[2]);
-                shift = table_shift(row[2]);
-                bias = row[3];
+    // One channel per thread (a slab has at most SLAB_CH = 128 channels, the block 256 threads): the weight-table
+    // row and the channel's weights are requested together, the workgroup then agrees on the PPE specialisation
+    // it runs (uniform), and the constants for it are written - one memory round trip before the main loop.
+    static_assert(NT >= SLAB_CH, "one channel per thread");
+    const int ch = threadIdx.x;
+    const bool has_ch = MODE != MODE_MAX && ch < nslab * 16;
+    int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0, wsum = 0;
+    if (has_ch) {
+        const int32_t c = box.z0 + slab0 * 16 + ch;
+        if (t.table != nullptr) {
+            const int32_t* row = t.table + (int64_t)c * t.table_stride;
+            mult = table_mult(row[2]);
+            shift = table_shift(row[2]);
+            bias = row[3];
+        }
+        if (MODE == MODE_DW) {
+            const uint8_t* row = t.weights + (int64_t)c * t.w_stride_oc;
+            for (int tap = 0; tap < ntaps; ++tap) {
+                const int32_t w = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
+                wsum += w;
+                s_w[tap * SLAB_CH + ch] = (float)w;
             }
-            bad_shift |= shift > kMaxF64Shift;
-            small_shift |= ppe_may_saturate((int64_t)ntaps * (MODE == MODE_DW ? 65025 : 255), bias, mult, shift);
+        } else {
+            wsum = ntaps;
         }
     }
+    const bool bad_shift = has_ch && shift > kMaxF64Shift;
+    const bool small_shift = has_ch && ppe_may_saturate((int64_t)ntaps * (MODE == MODE_DW ? 65025 : 255), bias, mult, shift);
     const bool use_int = __syncthreads_or(bad_shift) != 0;
     const bool may_sat = __syncthreads_or(small_shift) != 0;
     const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
     const int pmode = ppe_mode_of(pu, use_int);
-    if (MODE != MODE_MAX) {
-        for (int ch = threadIdx.x; ch < nslab * 16; ch += NT) {
-            const int32_t c = box.z0 + slab0 * 16 + ch;
-            int32_t wsum = 0;
-            if (MODE == MODE_DW) {
-                const uint8_t* row = t.weights + (int64_t)c * t.w_stride_oc;
-                for (int tap = 0; tap < ntaps; ++tap) {
-                    const int32_t w = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
-                    wsum += w;
-                    s_w[tap * SLAB_CH + ch] = (float)w;
-                }
-            } else {
-                wsum = ntaps;
-            }
-            int32_t mult = t.ppe.quant_mult, shift = t.ppe.quant_shift, bias = 0;
-            if (t.table != nullptr) {
-                const int32_t* row = t.table + (int64_t)c * t.table_stride;
-                mult = table_mult(row[2]);
-                shift = table_shift(row[2]);
-                bias = row[3];
-            }
-            // out-of-image taps were filled with the zero point: remove zpu * sum(w) exactly
-            const int32_t corr = -a.zpu * wsum;
-            sMult[ch] = mult;
-            sShift[ch] = shift;
-            sBias[ch] = bias;
-            sCorr[ch] = corr;  // |corr| < 2^23
-            const double M = ppe_scale_M(mult, shift);
-            sM[ch] = M;
-            sB[ch] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu);
-        }
+    if (has_ch) {
+        // out-of-image taps were filled with the zero point: remove zpu * sum(w) exactly
+        const int32_t corr = -a.zpu * wsum;
+        sMult[ch] = mult;
+        sShift[ch] = shift;
+        sBias[ch] = bias;
+        sCorr[ch] = corr;  // |corr| < 2^23
+        const double M = ppe_scale_M(mult, shift);
+        sM[ch] = M;
+        sB[ch] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu);
     }
     __syncthreads();
 
