@@ -487,3 +487,48 @@ def test_conv_wide_padded_kernel_on_chunked_kernel(executor):
     # 7x7 with padding over 64 channels fits LDS but needs more than 31 tap bits: row / column bits of the chunked kernel
     check(K.conv_case(512, 2, 13, 11, 64, 48, k=(7, 7), s=(1, 1), pads=(3, 3, 3, 3), in_zp=100), executor)
     check(K.conv_case(513, 1, 13, 11, 128, 32, k=(6, 6), s=(2, 2), pads=(2, 2, 3, 3), in_zp=7, w_signed=False, w_zp=131), executor)
+
+
+# ---- seeded random convolutions: kernel variants are picked by shape, so sweep shapes ---------------------------------
+
+def _random_conv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        ky, kx = (int(rng.integers(1, 6)), int(rng.integers(1, 6))) if rng.random() < 0.3 else (int(rng.choice([1, 3, 3, 5, 7])),) * 2
+        sy, sx = (int(rng.integers(1, 3)),) * 2 if rng.random() < 0.7 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        ic = int(rng.choice([16, 32, 48, 64, 64, 96, 128, 128, 192, 256, 320, 512]))
+        oc = int(rng.choice([16, 32, 48, 64, 80, 128, 144]))
+        pads = (int(rng.integers(0, kx // 2 + 1)), int(rng.integers(0, kx // 2 + 1)),   # left, right
+                int(rng.integers(0, ky // 2 + 1)), int(rng.integers(0, ky // 2 + 1)))   # top, bottom
+        h = int(rng.integers(max(ky, 3), 15))
+        w = int(rng.integers(max(kx, 3), 15))
+        n = int(rng.integers(1, 4))
+        in_signed = bool(rng.random() < 0.3)
+        w_signed = bool(rng.random() < 0.7)
+        in_zp = int(rng.integers(-128, 128)) if in_signed else int(rng.integers(0, 256))
+        w_zp = (0 if rng.random() < 0.6 else int(rng.integers(-20, 20))) if w_signed else (128 if rng.random() < 0.5 else int(rng.integers(100, 156)))
+        out_signed = bool(rng.random() < 0.3)
+        out_zp = int(rng.integers(-100, 100)) if out_signed else int(rng.integers(0, 200))
+        lo, hi = (-128, 127) if out_signed else (0, 255)   # clamp bounds in the output domain (after the zero point)
+        mode = rng.choice(["noop", "relu", "lrelu"])
+        if mode == "noop":
+            ppe = dict(mode=nce.PPE_NOOP, clamp_low=lo, clamp_high=hi)
+        elif mode == "relu":
+            ppe = dict(mode=nce.PPE_LRELU, clamp_low=max(lo, out_zp), clamp_high=hi)
+        else:
+            ppe = dict(mode=nce.PPE_LPRELU, clamp_low=lo, clamp_high=int(rng.integers(out_zp + 1, hi + 1)),
+                       lrelu_mult=int(rng.integers(1, 2048)), lrelu_shift=int(rng.integers(11, 16)))
+        cases.append(dict(seed=1000 + i, n=n, h=h, w=w, ic=ic, oc=oc, k=(ky, kx), s=(sy, sx), pads=pads,
+                          in_signed=in_signed, w_signed=w_signed, in_zp=in_zp, w_zp=w_zp, out_signed=out_signed, out_zp=out_zp, ppe=ppe))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(128, 20251), ids=lambda c: f"{c['n']}x{c['h']}x{c['w']}x{c['ic']}_{c['oc']}_k{c['k'][0]}x{c['k'][1]}s{c['s'][0]}x{c['s'][1]}")
+def test_conv_random_shapes(executor, case):
+    c = dict(case)
+    seed, n, h, w, ic, oc = (c.pop(k) for k in ("seed", "n", "h", "w", "ic", "oc"))
+    left, right, top, bottom = c["pads"]
+    if (h + top + bottom - c["k"][0]) // c["s"][0] + 1 < 1 or (w + left + right - c["k"][1]) // c["s"][1] + 1 < 1:
+        pytest.skip("window larger than the padded image")
+    check(K.conv_case(seed, n, h, w, ic, oc, **c), executor)
