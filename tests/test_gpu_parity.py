@@ -532,3 +532,36 @@ def test_conv_random_shapes(executor, case):
     if (h + top + bottom - c["k"][0]) // c["s"][0] + 1 < 1 or (w + left + right - c["k"][1]) // c["s"][1] + 1 < 1:
         pytest.skip("window larger than the padded image")
     check(K.conv_case(seed, n, h, w, ic, oc, **c), executor)
+
+
+def _random_window_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        kind = str(rng.choice(["dw", "max", "avg"]))
+        ky, kx = (int(rng.integers(1, 6)), int(rng.integers(1, 6))) if rng.random() < 0.4 else (int(rng.choice([2, 3, 3, 5])),) * 2
+        sy, sx = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pads = (int(rng.integers(0, kx // 2 + 1)), int(rng.integers(0, kx // 2 + 1)),
+                int(rng.integers(0, ky // 2 + 1)), int(rng.integers(0, ky // 2 + 1)))
+        c = 16 * int(rng.integers(1, 20))
+        h = int(rng.integers(max(ky, 3), 20))
+        w = int(rng.integers(max(kx, 3), 20))
+        n = int(rng.integers(1, 4))
+        in_signed = bool(rng.random() < 0.4)
+        in_zp = int(rng.integers(-128, 128)) if in_signed else int(rng.integers(0, 256))
+        cases.append(dict(kind=kind, seed=2000 + i, n=n, h=h, w=w, c=c, k=(ky, kx), s=(sy, sx), pads=pads, in_signed=in_signed, in_zp=in_zp,
+                          w_signed=bool(rng.random() < 0.6), w_zp=int(rng.integers(-10, 10)), with_table=bool(rng.random() < 0.5)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_window_cases(64, 777), ids=lambda c: f"{c['kind']}_{c['n']}x{c['h']}x{c['w']}x{c['c']}_k{c['k'][0]}x{c['k'][1]}s{c['s'][0]}x{c['s'][1]}")
+def test_window_random_shapes(executor, case):
+    c = dict(case)
+    kind, seed, n, h, w, ch = (c.pop(k) for k in ("kind", "seed", "n", "h", "w", "c"))
+    w_signed, w_zp, with_table = c.pop("w_signed"), c.pop("w_zp"), c.pop("with_table")
+    if kind == "dw":
+        zp = w_zp if w_signed else 128 + w_zp
+        check(K.dw_case(seed, n, h, w, ch, w_signed=w_signed, w_zp=zp, **c), executor)
+    else:
+        out_zp = 0 if kind == "max" else (c["in_zp"] // 2 if c["in_signed"] else 128 + c["in_zp"] // 4)
+        check(K.pool_case(seed, kind == "max", n, h, w, ch, with_table=with_table, out_zp=out_zp, **c), executor)
