@@ -617,16 +617,18 @@ hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t 
     // Transposed loads: measured to pay for every kernel larger than 1x1 and for long 1x1 reductions, once
     // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
     const bool trl = D >= 2 && mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
-    if constexpr (D == 2 || D == 4) {
+    if constexpr (D == 1 || D == 2 || D == 4) {
         if (w.a.dw != 0) {  // activation sums for the weight zero-point term
-            if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
-            if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
+            if constexpr (D >= 2) {
+                if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
+                if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TRL_ASUM>(w, nwaves, tpw, stream);
+            }
             if (mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
             if (mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
             return launch_one<NF, BF, WRES_GENERIC, D, LM_PLAIN_ASUM>(w, nwaves, tpw, stream);
         }
     }
-    if (w.a.dw != 0) return hipErrorNotSupported;  // (launch_mode sends those tasks to depth 2 or 4)
+    if (w.a.dw != 0) return hipErrorNotSupported;  // (launch_mode sends those tasks to depth 1, 2 or 4)
     if constexpr (D >= 2) {
         if (trl && mode == WRES_FAST) return launch_one<NF, BF, WRES_FAST, D, LM_TRL>(w, nwaves, tpw, stream);
         if (trl && mode == WRES_FAST_MASK) return launch_one<NF, BF, WRES_FAST_MASK, D, LM_TRL>(w, nwaves, tpw, stream);
@@ -643,8 +645,9 @@ hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t 
 template <int NF, int BF>
 hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
     if (w.a.dw != 0) {
-        // Depth 4 or 2 only. A padding step must read the fill line (its activations enter the pixel sums), which
-        // the mask mode guarantees: its tap bit is clear.
+        // Depth 4 or 2 only (1 for a single-step reduction). A padding step must read the fill line (its
+        // activations enter the pixel sums), which the mask mode guarantees: its tap bit is clear.
+        if (w.nsteps == 1) return launch_depth<NF, BF, 1>(w, mode, nwaves, tpw, stream);
         constexpr bool d4 = BF < 4;
         const bool pad = !(d4 && w.nsteps % 4 == 0) && w.nsteps % 2 != 0;
         if (pad && mode == WRES_FAST) {
