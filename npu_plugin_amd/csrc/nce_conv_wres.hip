@@ -27,7 +27,6 @@
 #include <cstdlib>
 
 namespace nce {
-namespace {
 
 struct WresArgs {
     ConvArgs a;
@@ -45,6 +44,15 @@ struct WresArgs {
     FastDiv div_nc64;   // by nc64
     int64_t row_adv;    // input offset from the last tap of a kernel row to the first of the next: in_sh - KX * in_sw
 };
+
+// This file is compiled twice (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
+// the 32-channel kernels and the chunked kernel, WRES_PART 1 the 64-channel kernels behind this entry point.
+#ifndef WRES_PART
+#define WRES_PART 0
+#endif
+hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream);
+
+namespace {
 
 enum { WRES_FAST = 0, WRES_FAST_MASK = 1, WRES_GENERIC = 2 };
 
@@ -669,6 +677,7 @@ hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t s
     return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
 }
 
+#if WRES_PART == 0
 // ---- reductions longer than LDS: the same kernel shape with the weights staged chunk by chunk ------------
 // For slices whose reduction does not fit LDS (3x3 over 1024 channels, 5x5 over 256, 1x1 over 8192 ...) the
 // workgroup stages CS steps of its weights, synchronises, lets every wave run those steps on its (single) tile,
@@ -995,6 +1004,8 @@ hipError_t launch_conv_wres_chunked(WresArgs& w, hipStream_t stream) {
     return bf == 2 ? launch_chunked<2, 2, false>(w, nw, stream) : launch_chunked<2, 1, false>(w, nw, stream);
 }
 
+#endif  // WRES_PART == 0
+
 template <int NF>
 hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream) {
     if (bf == 4) return launch_mode<NF, 4>(w, mode, nwaves, tpw, stream);
@@ -1004,6 +1015,11 @@ hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStre
 
 }  // namespace
 
+#if WRES_PART == 1
+hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream) {
+    return launch_bf<4>(w, bf, mode, nwaves, tpw, stream);
+}
+#else
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked) {
     if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
@@ -1058,8 +1074,9 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
             if (ftpw >= 1) tpw = ftpw;
         }
     }
-    if (nf == 4) return launch_bf<4>(w, bf, mode, nw, tpw, stream);
+    if (nf == 4) return launch_wres_nf4(w, bf, mode, nw, tpw, stream);
     return launch_bf<2>(w, bf, mode, nw, tpw, stream);
 }
+#endif  // WRES_PART
 
 }  // namespace nce
