@@ -565,3 +565,28 @@ def test_window_random_shapes(executor, case):
     else:
         out_zp = 0 if kind == "max" else (c["in_zp"] // 2 if c["in_signed"] else 128 + c["in_zp"] // 4)
         check(K.pool_case(seed, kind == "max", n, h, w, ch, with_table=with_table, out_zp=out_zp, **c), executor)
+
+
+def _random_eltwise_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        signed = bool(rng.random() < 0.4)
+        zp = (lambda: int(rng.integers(-128, 128))) if signed else (lambda: int(rng.integers(0, 256)))
+        mult = int(rng.integers(8192, 65536))
+        shift = int(rng.integers(18, 36))
+        extra = {}
+        if rng.random() < 0.3:
+            extra = dict(mode=nce.PPE_LPRELU, lrelu_mult=int(rng.integers(1, 2048)), lrelu_shift=int(rng.integers(11, 16)))
+        cases.append(dict(seed=3000 + i, n=int(rng.integers(1, 4)), h=int(rng.integers(1, 17)), w=int(rng.integers(1, 17)),
+                          c=16 * int(rng.integers(1, 24)), signed=signed, zp_a=zp(), zp_b=zp(), out_zp=zp(),
+                          in1_mult=int(rng.integers(1, 65536)), in2_mult=int(rng.integers(1, 65536)), mult=mult, shift=shift,
+                          with_in_mult=bool(rng.random() < 0.8), with_table=bool(rng.random() < 0.25), ppe_extra=extra or None))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_eltwise_cases(48, 4242), ids=lambda c: f"{c['n']}x{c['h']}x{c['w']}x{c['c']}_{'i8' if c['signed'] else 'u8'}_s{c['shift']}")
+def test_eltwise_random(executor, case):
+    c = dict(case)
+    seed, n, h, w, ch = (c.pop(k) for k in ("seed", "n", "h", "w", "c"))
+    check(K.eltwise_case(seed, n, h, w, ch, **c), executor)
