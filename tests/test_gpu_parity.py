@@ -590,3 +590,15 @@ def test_eltwise_random(executor, case):
     c = dict(case)
     seed, n, h, w, ch = (c.pop(k) for k in ("seed", "n", "h", "w", "c"))
     check(K.eltwise_case(seed, n, h, w, ch, **c), executor)
+
+
+def test_conv_long_reduction_and_weight_zero_point_variants(executor):
+    # sub-boxes (workloads) on the chunked kernel and on the kernels with pixel sums
+    for kw in (dict(ic=256, k=(5, 5), pads=(2, 2, 2, 2)), dict(ic=128, k=(3, 3), pads=(1, 1, 1, 1), w_signed=False, w_zp=121),
+               dict(ic=64, k=(1, 1), pads=(0, 0, 0, 0), w_signed=True, w_zp=-4)):
+        ic = kw.pop("ic")
+        full = K.conv_case(910 + ic, 2, 12, 10, ic, 64, **kw)
+        want = K.run_oracle(full)
+        tiled = K.conv_case(910 + ic, 2, 12, 10, ic, 64, variants=[((0, 0, 0), (9, 5, 31)), ((0, 6, 0), (9, 11, 31)),
+                                                                    ((0, 0, 32), (4, 11, 63)), ((5, 0, 32), (9, 11, 63))], **kw)
+        assert np.array_equal(K.run_hip(tiled, executor), want)
