@@ -216,7 +216,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     __shared__ int32_t sCorr[8][OCT];   // integer path: da * sum of weights
     __shared__ double sBfull[8][OCT];   // FP64 paths: bias term + da * M * sum of weights (+ output zero point)
     __shared__ int32_t sFlags;
-    __shared__ StepEntry sStep[kMaxSteps];
+    __shared__ StepEntry sStep[MODE == WRES_GENERIC ? 4 * kMaxSteps : kMaxSteps];  // per-lane mode: one entry per 16-byte unit
     const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
 
     const int tid = threadIdx.x;
@@ -313,20 +313,33 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         e.pad = 0;
         return e;
     };
+    // Per-lane mode: entry of 16-byte unit u of the reduction - input offset, bit of its kernel row (tap_bit)
+    // and of its kernel column (pad). Units past the reduction's end have no bits: they read the fill value.
+    auto unit_entry = [&](int u) {
+        const int tap = fdiv(u, w.div_icg);
+        const int icg = u - tap * a.ICG;
+        const int ky = fdiv(tap, w.div_kx);
+        const int kx = tap - ky * a.KX;
+        const bool real = u < w.k16;
+        const int64_t off = real ? (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + icg * 16 : 0;
+        StepEntry e;
+        e.off_lo = (int32_t)(uint32_t)off;
+        e.off_hi = (int32_t)(off >> 32);
+        e.tap_bit = real ? 1u << ky : 0u;
+        e.pad = real ? 1u << kx : 0u;
+        return e;
+    };
     // Request the activation operand of the next step for every pixel fragment (raw bytes). The table of
     // steps is valid after the workgroup's barrier; the first tile's first requests go out before it and
     // compute their entries (from_table = false).
     auto load_b = [&](v4i (&d)[BF], bool from_table = true) {
         if (MODE == WRES_GENERIC) {
             const int u = 4 * ls + kc;
-            const int tap = fdiv(u, w.div_icg);
-            const int icg = u - tap * a.ICG;
-            const int ky = fdiv(tap, w.div_kx);
-            const int kx = tap - ky * a.KX;
-            const int64_t off = (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + icg * 16;
+            const StepEntry e = from_table ? sStep[u] : unit_entry(u);
+            const int64_t off = ((int64_t)e.off_hi << 32) | (uint32_t)e.off_lo;
 #pragma unroll
             for (int x = 0; x < BF; ++x) {
-                const bool ok = u < w.k16 && ((mask0[x] >> ky) & (mask1[x] >> kx) & 1u) != 0;
+                const bool ok = (mask0[x] & e.tap_bit) != 0 && (mask1[x] & e.pad) != 0;
                 const uint8_t* src = ok ? pbase[x] + off : fillp;
                 d[x] = *reinterpret_cast<const v4i*>(src);
             }
@@ -485,6 +498,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     }
     if constexpr (TBL) {
         for (int st = tid; st < S; st += (int)blockDim.x) sStep[st] = step_entry(st);
+    } else if (MODE == WRES_GENERIC) {
+        for (int u = tid; u < 4 * S; u += (int)blockDim.x) sStep[u] = unit_entry(u);
     }
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
 
@@ -613,6 +628,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     w.nsteps = (w.nsteps + D - 1) / D * D;
     const size_t lds = (size_t)w.nsteps * NF * 1024;
     if (lds > kWresLdsCap || w.nsteps > kMaxSteps) return hipErrorNotSupported;
+    if (MODE == WRES_GENERIC && lds > kWresLdsCap - 4096) return hipErrorNotSupported;  // its step table is 4 KiB larger
     auto kernel = &conv_wres_kernel<NF, BF, MODE, D, LM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
