@@ -101,6 +101,8 @@ struct EpiPack {
     uint32_t flip;      // 0x80808080 for signed outputs
     double zp_fold;     // what B carries on top of the bias term: the output zero point (+128 for signed outputs)
     double pcz;         // slope mode: rounding constant of the slope + zp_fold * (1 - slope)
+    int32_t pmq;        // high-word slope mode: slope * 2^32 ...
+    int64_t cpz;        // ... and (rounding constant + zp_fold * (1 - slope)) * 2^32
 };
 
 __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
@@ -111,6 +113,8 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     e.flip = sb ? 0x80808080u : 0u;
     e.zp_fold = (double)(pu.zp + sb);
     e.pcz = pu.pc + e.zp_fold - e.zp_fold * pu.pm;  // exact: 8 integer bits, at most 31 fractional bits
+    e.pmq = 0;
+    e.cpz = 0;
     return e;
 }
 
@@ -132,10 +136,15 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
             double M = 0.0, B = 0.0;
             int32_t w2 = 0, bias = 0, corr = 0;
             // (the activation zero point is already in the wave's constants: da * sum of the channel's weights)
+            int32_t mq = 0;
+            int64_t cq = 0;
             if (PMODE == PPE_MODE_INT) {
                 w2 = s.w2[c];
                 bias = s.bias[c];
                 corr = sCorr[c];
+            } else if (PMODE == PPE_MODE_HI || PMODE == PPE_MODE_HI_SLOPE) {
+                mq = sCorr[c];
+                cq = reinterpret_cast<const int64_t*>(sBfull)[c];
             } else {
                 M = s.M[c];
                 B = sBfull[c];
@@ -146,6 +155,20 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
                 if (PMODE == PPE_MODE_INT) {
                     const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
                     wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
+                } else if (PMODE == PPE_MODE_HI) {
+                    // y = floor(((av + bias') * mult + 2^(shift-1) + zp * 2^shift) / 2^shift), everything scaled
+                    // by 2^(32 - shift) so that the division is "take the high word": one 32 x 32 + 64 bit
+                    // multiply-add per output. mq and cq are set up per wave (see kernel).
+                    const int32_t y = clamp_med3((int32_t)(((int64_t)av * mq + cq) >> 32), ep.ilo, ep.ihi);
+                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
+                } else if (PMODE == PPE_MODE_HI_SLOPE) {
+                    // The same with a negative slope |slope| <= 1: rz is the value before the slope (zero point
+                    // added), nz the value after it, both exact; the larger of the two is the result (below
+                    // zero the slope raises a value, from zero up it does not).
+                    const int32_t rz = (int32_t)(((int64_t)av * mq + cq) >> 32);
+                    const int32_t nz = (int32_t)(((int64_t)rz * ep.pmq + ep.cpz) >> 32);
+                    const int32_t y = min(max(max(rz, nz), ep.ilo), ep.ihi);
+                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
                 } else if (PMODE == PPE_MODE_FOLDED) {
                     // The conversion truncates; below zero that differs from floor, but every value below
                     // zero (and floor's -1 for a value in (-1, 0)) clamps to ep.ilo >= 0 either way.
@@ -408,7 +431,15 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t mult = table_mult(tw2), shift = table_shift(tw2);
             const bool bad = lane < OCT && shift > kMaxF64Shift;
             const bool sat = lane < OCT && ppe_may_saturate(acc_bound, tbias, mult, shift);
-            const int wf = (__any(bad) ? 1 : 0) | (__any(sat) ? 2 : 0);
+            // High-word integer epilogue: needs mult * 2^(32 - shift) in int32 and the 64-bit constant (bias and
+            // weight-sum terms, below 2^32 together, times the scale; rounding and zero-point terms) below 2^62.
+            bool hi_bad = false;
+            if (lane < noc) {
+                hi_bad = shift < 1 || shift > 32 || ((int64_t)mult << (32 - min(shift, 32))) > 0x7fffffffLL;
+                const double cb = ((__builtin_fabs((double)tbias) + 4294967296.0) * (double)mult + 2147483648.0 + 384.0 * __builtin_ldexp(1.0, shift));
+                hi_bad = hi_bad || __builtin_ldexp(cb, 32 - shift) >= 4611686018427387904.0;
+            }
+            const int wf = (__any(bad) ? 1 : 0) | (__any(sat) ? 2 : 0) | (__any(hi_bad) ? 4 : 0);
             if (lane == 0) sFlags = wf;
             if (lane < OCT) {
                 const double M = ppe_scale_M(mult, shift);
@@ -505,8 +536,25 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
 
     const int flags = sFlags;
     const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
-    const int pmode = ppe_mode_of(pu, (flags & 1) != 0);
-    const EpiPack ep = epi_pack_setup(pu);
+    int pmode = ppe_mode_of(pu, (flags & 1) != 0);
+    if (pmode == PPE_MODE_FOLDED && !(flags & 4)) pmode = PPE_MODE_HI;
+    EpiPack ep = epi_pack_setup(pu);
+    if (pmode == PPE_MODE_SLOPE && !(flags & 4)) {
+        // slope = pm * 2^-ps with |slope| <= 1 in this mode; the high-word form needs slope * 2^32 in int32
+        const int32_t pm = a.ppe.prelu_mult, ps = a.ppe.prelu_shift;
+        if (ps <= 32 && (ps >= 1 || pm == 0)) {
+            const int64_t q = (int64_t)pm * ((int64_t)1 << (32 - ps));
+            if (q >= -0x7fffffffLL && q <= 0x7fffffffLL) {
+                const int64_t zpf = pu.zp + (ep.flip ? 128 : 0);
+                const int64_t half = ps >= 1 ? (int64_t)1 << (ps - 1) : 0;
+                pmode = PPE_MODE_HI_SLOPE;
+                // (through readfirstlane: otherwise the compiler replaces the sign-extended 32-bit value by the 64-bit q
+                // it was cut from and multiplies 64 x 64 bits per output)
+                ep.pmq = __builtin_amdgcn_readfirstlane((int32_t)q);
+                ep.cpz = (half + zpf * ((int64_t)1 << ps) - zpf * pm) * ((int64_t)1 << (32 - ps));
+            }
+        }
+    }
     // This wave's copy of the per-channel constants with the weight sums folded in (lane = channel). The
     // activation zero point enters as da * (sum of the channel's weights): |da| <= 255, |sum| < 2^23, and
     // the FP64 product and sum are exact (24 x 25 significant bits).
@@ -520,6 +568,19 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         if (ASUM) B = __builtin_fma((double)kdd, sM[lane], B);
         if (pmode != PPE_MODE_INT) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
         sBfull[wave][lane] = B;
+        if (pmode == PPE_MODE_HI || pmode == PPE_MODE_HI_SLOPE) {
+            const int32_t mult = table_mult(sW2[lane]), shift = table_shift(sW2[lane]);
+            int32_t mq = 0;
+            int64_t cq = 0;
+            if (lane < noc) {  // (channels past the slice's end keep zeros; their results are not stored)
+                const int64_t base = ((int64_t)sBias[lane] + sCorr[wave][lane]) * mult + ((int64_t)1 << (shift - 1))
+                                   + ((int64_t)(pu.zp + (ep.flip ? 128 : 0)) << shift);
+                mq = (int32_t)((uint32_t)mult << (32 - shift));
+                cq = (int64_t)((uint64_t)base << (32 - shift));
+            }
+            sCorr[wave][lane] = mq;
+            reinterpret_cast<int64_t*>(sBfull[wave])[lane] = cq;
+        }
     }
     // (same wave writes and reads: program order is enough, the compiler waits on the LDS counter)
 
@@ -603,7 +664,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         int32_t dws[BF];  // every row of asum holds the pixel's sum: register 0 of this lane is its column's
 #pragma unroll
         for (int x = 0; x < BF; ++x) dws[x] = ASUM ? a.dw * asum[x][0] : 0;
-        if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        if (pmode == PPE_MODE_HI) wres_epilogue<NF, BF, PPE_MODE_HI>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_HI_SLOPE) wres_epilogue<NF, BF, PPE_MODE_HI_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        else if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
         else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
         else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
         t += nwaves;
@@ -622,7 +685,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     constexpr int BP = 16 * BF;
     const ConvArgs& a = w.a;
     w.ntiles = (uint32_t)(((int64_t)a.M + BP - 1) / BP);
-    w.tpg = nwaves * tiles_per_wave;
+    if (w.tpg == 0) w.tpg = nwaves * tiles_per_wave;  // (the caller may have chosen a tile count per workgroup that is no multiple)
     w.ngroups = (w.ntiles + w.tpg - 1) / w.tpg;
     const unsigned gy = (unsigned)((a.bc + OCT - 1) / OCT);
     w.nsteps = (w.nsteps + D - 1) / D * D;
@@ -1077,7 +1140,15 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     while (bf > 1 && wave_tiles(nf, bf) < want) bf >>= 1;
     if (nf == 4 && wave_tiles(nf, bf) < want) nf = 2;
     const int nwaves = 8;
-    int tpw = (int)std::max<int64_t>(1, wave_tiles(nf, bf) / 1568);
+    int tpw = 1;
+    // Tiles per workgroup: one workgroup per CU where the tiles reach that far (the waves of a workgroup then
+    // take unequal numbers of tiles, which costs less than leaving CUs idle or queueing a second round).
+    const auto pick_tpg = [&](int nf_, int bf_, int nw_) {
+        const int64_t ntiles = ((int64_t)a.M + 16 * bf_ - 1) / (16 * bf_);
+        const int64_t slices = (a.bc + 16 * nf_ - 1) / (16 * nf_);
+        const int64_t groups = std::max<int64_t>(1, 256 / slices);
+        return (uint32_t)std::max<int64_t>(nw_, (ntiles + groups - 1) / groups);
+    };
 
     int nw = nwaves;
     const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning and test knob: "nf,bf,nwaves,tiles_per_wave"
@@ -1090,6 +1161,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
             if (ftpw >= 1) tpw = ftpw;
         }
     }
+    w.tpg = forced ? 0 : pick_tpg(nf, bf, nw);
     if (nf == 4) return launch_wres_nf4(w, bf, mode, nw, tpw, stream);
     return launch_bf<2>(w, bf, mode, nw, tpw, stream);
 }

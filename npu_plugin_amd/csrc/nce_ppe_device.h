@@ -146,7 +146,9 @@ __device__ __forceinline__ int32_t ppe_finish_f64_folded(double v, int32_t lo_zp
 // Which specialisation a workgroup runs (uniform). FOLDED and SLOPE cover rounding half-up without
 // int32 saturation (every shift >= 18), with or without a negative slope; every other combination
 // (ties-to-even, floor, tiny shifts, slopes that can overflow) runs the integer path.
-enum { PPE_MODE_FOLDED = 0, PPE_MODE_SLOPE = 1, PPE_MODE_INT = 3 };
+// (PPE_MODE_HI, PPE_MODE_HI_SLOPE: the folded and slope modes in 64-bit integer arithmetic; a kernel that sets
+// up their constants opts in.)
+enum { PPE_MODE_FOLDED = 0, PPE_MODE_SLOPE = 1, PPE_MODE_INT = 3, PPE_MODE_HI = 4, PPE_MODE_HI_SLOPE = 5 };
 
 __device__ __forceinline__ int ppe_mode_of(const PpeF64& u, bool use_int) {
     if (use_int || u.even || u.sat || u.round_none) return PPE_MODE_INT;
