@@ -1135,10 +1135,11 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
         return (((int64_t)a.M + 16 * bf - 1) / (16 * bf)) * ((a.bc + 16 * nf - 1) / (16 * nf));
     };
     const bool nf4_ok = wl4 <= kWresLdsCap && a.bc > 32;
-    const int64_t want = 1500;
+    // (1x1 kernels over more than 64 input channels: measured faster with smaller pixel tiles, about 24 per CU)
+    const int64_t want = (w.ntaps == 1 && w.nsteps > 1) ? 6000 : 1500;
     int nf = nf4_ok ? 4 : 2, bf = 4;
     while (bf > 1 && wave_tiles(nf, bf) < want) bf >>= 1;
-    if (nf == 4 && wave_tiles(nf, bf) < want) nf = 2;
+    if (nf == 4 && wave_tiles(nf, bf) < 1500) nf = 2;
     const int nwaves = 8;
     int tpw = 1;
     // Tiles per workgroup: one workgroup per CU where the tiles reach that far (the waves of a workgroup then
@@ -1151,6 +1152,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     };
 
     int nw = nwaves;
+    bool forced_tpw = false;
     const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning and test knob: "nf,bf,nwaves,tiles_per_wave"
     if (forced) {
         int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
@@ -1158,10 +1160,10 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
             if ((fnf == 2 || (fnf == 4 && wl4 <= kWresLdsCap))) nf = fnf;
             if (fbf == 1 || fbf == 2 || fbf == 4) bf = fbf;
             if (fnw >= 1 && fnw <= 8) nw = fnw;
-            if (ftpw >= 1) tpw = ftpw;
+            if (ftpw >= 1) tpw = ftpw, forced_tpw = true;  // (0: keep the automatic choice below)
         }
     }
-    w.tpg = forced ? 0 : pick_tpg(nf, bf, nw);
+    w.tpg = forced_tpw ? 0 : pick_tpg(nf, bf, nw);
     if (nf == 4) return launch_wres_nf4(w, bf, mode, nw, tpw, stream);
     return launch_bf<2>(w, bf, mode, nw, tpw, stream);
 }
