@@ -43,6 +43,9 @@ struct WresArgs {
     FastDiv div_kx;     // by KX
     FastDiv div_nc64;   // by nc64
     int64_t row_adv;    // input offset from the last tap of a kernel row to the first of the next: in_sh - KX * in_sw
+    // The tensor strides once more as 32-bit values (the host checks that they fit): index * stride is then one
+    // 32 x 32 + 64 bit multiply-add instead of a 64-bit multiplication.
+    int32_t in_sn32, in_sh32, in_sw32, out_sn32, out_sh32, out_sw32;
 };
 
 // This file is compiled twice (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
@@ -282,9 +285,9 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t pc = valid[x] ? (int32_t)p : a.M - 1;  // lanes past the end compute a duplicate
             if (w.linear) {  // uniform: no decomposition into image, row and column
                 const uint32_t ps = t * BP + 16 * x + c16;  // pixel this lane holds in matrix layout
-                pbase[x] = a.in + (int64_t)pc * a.in_sw + (MODE == WRES_GENERIC ? 0 : kc * 16);
+                pbase[x] = a.in + (int64_t)pc * w.in_sw32 + (MODE == WRES_GENERIC ? 0 : kc * 16);
                 valid[x] = ps < (uint32_t)a.M;
-                dst[x] = a.out + (int64_t)(valid[x] ? (int32_t)ps : a.M - 1) * a.out_sw + oc0 * a.out_sc;
+                dst[x] = a.out + (int64_t)(valid[x] ? (int32_t)ps : a.M - 1) * w.out_sw32 + oc0 * a.out_sc;
                 mask0[x] = mask1[x] = 1;
                 continue;
             }
@@ -294,8 +297,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
             const int32_t by = rr - n * a.bh;
             const int32_t iy0 = (a.y0 + by) * a.SY - a.PT;
             const int32_t ix0 = (a.x0 + bx) * a.SX - a.PL;
-            pbase[x] = a.in + (int64_t)n * a.in_sn + (int64_t)iy0 * a.in_sh + (int64_t)ix0 * a.in_sw + (MODE == WRES_GENERIC ? 0 : kc * 16);
-            dst[x] = a.out + (int64_t)n * a.out_sn + (int64_t)(a.y0 + by) * a.out_sh + (int64_t)(a.x0 + bx) * a.out_sw + oc0 * a.out_sc;
+            pbase[x] = a.in + (int64_t)n * w.in_sn32 + (int64_t)iy0 * w.in_sh32 + (int64_t)ix0 * w.in_sw32 + (MODE == WRES_GENERIC ? 0 : kc * 16);
+            dst[x] = a.out + (int64_t)n * w.out_sn32 + (int64_t)(a.y0 + by) * w.out_sh32 + (int64_t)(a.x0 + bx) * w.out_sw32 + oc0 * a.out_sc;
             if (TRL) {  // results come out in matrix layout: take the address of pixel c16 from a lane that computed it
                 const uint64_t dl = reinterpret_cast<uint64_t>(dst[x]);
                 const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(16 * c16, (int)(uint32_t)dl);
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         const int ky = fdiv(tap, w.div_kx);
         const int kx = tap - ky * a.KX;
         const bool real = tap < w.ntaps;  // padding steps stay on a readable address, their tap bit is clear
-        const int64_t off = real ? (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + c64 * 64 : 0;
+        const int64_t off = real ? (int64_t)ky * w.in_sh32 + (int64_t)kx * w.in_sw32 + c64 * 64 : 0;
         StepEntry e;
         e.off_lo = (int32_t)(uint32_t)off;
         e.off_hi = (int32_t)(off >> 32);
@@ -344,7 +347,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         const int ky = fdiv(tap, w.div_kx);
         const int kx = tap - ky * a.KX;
         const bool real = u < w.k16;
-        const int64_t off = real ? (int64_t)ky * a.in_sh + (int64_t)kx * a.in_sw + icg * 16 : 0;
+        const int64_t off = real ? (int64_t)ky * w.in_sh32 + (int64_t)kx * w.in_sw32 + icg * 16 : 0;
         StepEntry e;
         e.off_lo = (int32_t)(uint32_t)off;
         e.off_hi = (int32_t)(off >> 32);
@@ -1113,6 +1116,14 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     w.div_kx = make_fastdiv((uint32_t)a.KX);
     w.div_nc64 = make_fastdiv((uint32_t)std::max(1, w.nc64));
     w.row_adv = a.in_sh - (int64_t)a.KX * a.in_sw;
+    for (const int64_t st : {a.in_sn, a.in_sh, a.in_sw, a.out_sn, a.out_sh, a.out_sw})
+        if (st < 0 || st > 0x7fffffffLL) return hipErrorNotSupported;
+    w.in_sn32 = (int32_t)a.in_sn;
+    w.in_sh32 = (int32_t)a.in_sh;
+    w.in_sw32 = (int32_t)a.in_sw;
+    w.out_sn32 = (int32_t)a.out_sn;
+    w.out_sh32 = (int32_t)a.out_sh;
+    w.out_sw32 = (int32_t)a.out_sw;
     const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
     if (wl2 > kWresLdsCap) return allow_chunked ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
 
