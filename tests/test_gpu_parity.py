@@ -602,3 +602,50 @@ def test_conv_long_reduction_and_weight_zero_point_variants(executor):
         tiled = K.conv_case(910 + ic, 2, 12, 10, ic, 64, variants=[((0, 0, 0), (9, 5, 31)), ((0, 6, 0), (9, 11, 31)),
                                                                     ((0, 0, 32), (4, 11, 63)), ((5, 0, 32), (9, 11, 63))], **kw)
         assert np.array_equal(K.run_hip(tiled, executor), want)
+
+
+def _table_with(case, mults, shifts, biases):
+    """Overwrite words [2] and [3] of the case's weight table, cycling through the given values per channel."""
+    t = case.table.astype(np.int64)
+    for c in range(t.shape[0]):
+        t[c, 2] = (int(mults[c % len(mults)]) << 16) | (int(shifts[c % len(shifts)]) << 8)
+        t[c, 3] = int(biases[c % len(biases)])
+    case.table = (t & 0xFFFFFFFF).astype(np.uint32).view(np.int32).reshape(-1, 4).copy()
+    return case
+
+
+HI_SLOPES = [dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255),
+             dict(mode=nce.PPE_LRELU, clamp_low=0, clamp_high=255),                                    # slope 0
+             dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1023, lrelu_shift=11),  # just below 1/2
+             dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1, lrelu_shift=1),      # 1/2: FP64 path
+             dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=3, lrelu_shift=2),      # 3/4: FP64 path
+             dict(mode=nce.PPE_LPRELU, clamp_low=3, clamp_high=250, lrelu_mult=1, lrelu_shift=31)]
+
+
+@pytest.mark.parametrize("ppe", HI_SLOPES, ids=lambda p: f"m{p.get('lrelu_mult', '-')}s{p.get('lrelu_shift', '-')}")
+@pytest.mark.parametrize("shift", [1, 15, 16, 17, 24, 31, 32, 33, 40])
+def test_conv_epilogue_shift_boundaries(executor, ppe, shift):
+    # Every channel of a slice with the same shift: the integer high-word epilogue serves 16/17..32 (the multiplier
+    # must fit 31 bits after scaling), FP64 or the 64-bit integer path the rest. Multipliers and biases at their
+    # extremes; small shifts saturate.
+    for out_signed, out_zp in ((False, 128), (True, -7), (False, 0)):
+        lo, hi = (-128, 127) if out_signed else (0, 255)
+        p = dict(ppe, clamp_low=max(lo, ppe["clamp_low"] + lo), clamp_high=min(hi, ppe["clamp_high"] + lo))
+        case = K.conv_case(4000 + shift, 1, 9, 9, 64, 64, k=(1, 1), pads=(0, 0, 0, 0), ppe=p, out_signed=out_signed,
+                           out_zp=out_zp)
+        scale = 2.0 ** (shift - 22)   # keeps a part of the outputs inside the clamp range for every shift
+        biases = [0, 1, -1, int(1000 * scale), -int(900 * scale), 2**31 - 1, -2**31, int(2**20 * scale), -int(2**20 * scale)]
+        biases = [max(-2**31, min(2**31 - 1, b)) for b in biases]
+        check(_table_with(case, [1, 16384, 32767, 65535, 0, 40000, 12345], [shift], biases), executor)
+
+
+def test_conv_epilogue_mixed_shifts_in_one_slice(executor):
+    # One channel outside the high-word range sends its whole slice to the FP64 epilogue; the other slice stays.
+    case = K.conv_case(4100, 2, 7, 7, 128, 128, k=(3, 3), pads=(1, 1, 1, 1),
+                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14))
+    t = case.table.astype(np.int64)
+    t[70, 2] = (20000 << 16) | (35 << 8)
+    t[71, 2] = (65535 << 16) | (16 << 8)
+    t[72, 3] = 2**31 - 1
+    case.table = (t & 0xFFFFFFFF).astype(np.uint32).view(np.int32).reshape(-1, 4).copy()
+    check(case, executor)
