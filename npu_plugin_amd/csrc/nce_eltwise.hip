@@ -27,10 +27,19 @@ struct EltArgs {
     // the packed word; B carries the output zero point and that 128), clamp bounds in that domain
     int32_t ilo, ihi;
     uint32_t flip;
+    // high-word path: the folded path in integers. y = high word of acc * mq + cq with mq = quant_mult * 2^(32 - shift)
+    // and cq = (2^(shift-1) + zero point * 2^shift) * 2^(32 - shift); acc = in1_mult * a + in2_mult * b + c0h as one
+    // unsigned 16-bit dot product (signed inputs enter 128 higher, c0h takes that back).
+    int32_t mq, c0h;
+    int64_t cq;
+    uint32_t mults;     // in1_mult | in2_mult << 16
+    uint32_t in_flip;   // 0x80808080 for signed inputs
 };
 
-// PATH = a PPE_MODE_* value with uniform scale, or PATH_TABLE: integer with a per-channel table.
+// PATH = a PPE_MODE_* value with uniform scale, PATH_TABLE: integer with a per-channel table, or PATH_HI.
 constexpr int PATH_TABLE = 4;
+constexpr int PATH_HI = 5;
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 template <bool FLAT, int PATH, bool SIGNED>
 __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
@@ -64,6 +73,23 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
         const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
         const uint32_t wb[4] = {vb.x, vb.y, vb.z, vb.w};
         uint32_t wo[4];
+        if (PATH == PATH_HI) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t ua = wa[d] ^ a.in_flip, ub = wb[d] ^ a.in_flip;
+                uint32_t packed = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // bytes i of a and b, zero-extended to a pair of 16-bit values: 0x0c selects a zero byte
+                    const uint32_t pair = __builtin_amdgcn_perm(ub, ua, 0x0c040c00u + (uint32_t)i * 0x00010001u);
+                    const int32_t acc = (int32_t)__builtin_amdgcn_udot2(__builtin_bit_cast(u16x2, pair), __builtin_bit_cast(u16x2, a.mults),
+                                                                         (uint32_t)a.c0h, false);
+                    const int32_t y = clamp_med3((int32_t)(((int64_t)acc * a.mq + a.cq) >> 32), a.ilo, a.ihi);
+                    packed = i == 0 ? (uint32_t)y : (packed | ((uint32_t)y << (8 * i)));
+                }
+                wo[d] = packed ^ a.flip;
+            }
+        } else
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             uint32_t packed = 0;
@@ -107,6 +133,7 @@ void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
     if (path == PPE_MODE_FOLDED) launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
     else if (path == PPE_MODE_SLOPE) launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
     else if (path == PPE_MODE_INT) launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
+    else if (path == PATH_HI) hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH_HI, false>), dim3(grid), dim3(256), 0, s, a);
     else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
 
@@ -137,6 +164,9 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     else path = prelu ? PPE_MODE_SLOPE : PPE_MODE_FOLDED;
     a.ilo = a.ihi = 0;
     a.flip = 0;
+    a.mq = a.c0h = 0;
+    a.cq = 0;
+    a.mults = a.in_flip = 0;
     if (path == PPE_MODE_FOLDED) {
         const int32_t lo_zp = t.ppe.lo + t.ppe.zp_out, hi_zp = t.ppe.hi + t.ppe.zp_out;
         const int32_t sb = lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
@@ -144,6 +174,17 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
         a.ilo = lo_zp + sb;
         a.ihi = hi_zp + sb;
         a.flip = sb ? 0x80808080u : 0u;
+        // The integer form of the same: multiplier scaled to 2^32 must fit int32, input multipliers 16 bits.
+        const int64_t mq = (shift >= 1 && shift <= 32) ? (int64_t)t.ppe.quant_mult << (32 - shift) : -1;
+        if (mq >= 0 && mq <= 0x7fffffffLL && t.ppe.in1_mult >= 0 && t.ppe.in1_mult <= 65535 && t.ppe.in2_mult >= 0 &&
+            t.ppe.in2_mult <= 65535) {
+            path = PATH_HI;
+            a.mq = (int32_t)mq;
+            a.cq = (((int64_t)1 << (shift - 1)) << (32 - shift)) + ((int64_t)(t.ppe.zp_out + sb) << 32);
+            a.mults = (uint32_t)t.ppe.in1_mult | ((uint32_t)t.ppe.in2_mult << 16);
+            a.in_flip = t.in.is_signed ? 0x80808080u : 0u;
+            a.c0h = a.c0 - (t.in.is_signed ? 128 * (t.ppe.in1_mult + t.ppe.in2_mult) : 0);
+        }
     }
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;

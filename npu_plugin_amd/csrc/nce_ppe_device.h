@@ -7,8 +7,8 @@
 //
 // Two implementations of the same function:
 //   * ppe_apply      - 64-bit integer arithmetic, any shift 0..63.
-//   * ppe_apply_f64  - the same value through FP64, which gfx950 issues at full rate while 64-bit
-//                      integer multiplies and shifts do not. Exact, not approximate: with
+//   * ppe_apply_f64  - the same value through FP64 (gfx950 issues FP64 FMA and conversions at the 32-bit
+//                      rate; a general 64-bit shift-and-round takes several instructions). Exact, not approximate: with
 //                      M = mult * 2^-shift and B = bias * M + 1/2, the quantity acc * M + B equals
 //                      N / 2^shift for an integer |N| < 2^53 whenever shift <= 52, so one FMA
 //                      returns it without rounding and floor() (or rint() for ties-to-even) is the
