@@ -649,3 +649,15 @@ def test_conv_epilogue_mixed_shifts_in_one_slice(executor):
     t[72, 3] = 2**31 - 1
     case.table = (t & 0xFFFFFFFF).astype(np.uint32).view(np.int32).reshape(-1, 4).copy()
     check(case, executor)
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("shift,mult", [(17, 65535), (17, 40000), (16, 32767), (16, 40000), (24, 1), (32, 65535), (33, 65535),
+                                        (31, 16384), (26, 0)])
+def test_eltwise_integer_path_boundaries(executor, signed, shift, mult):
+    # the high-word form serves shifts up to 32 whose scaled multiplier fits 31 bits; input multipliers at both ends
+    for in1, in2 in ((65535, 65535), (1, 65535), (0, 1), (20971, 31457)):
+        # pick the input multipliers' common scale so that sums stay inside the output range for a part of the inputs
+        zp = -5 if signed else 128
+        check(K.eltwise_case(5000 + shift, 2, 5, 7, 48, signed=signed, zp_a=zp, zp_b=zp + 3, out_zp=zp, in1_mult=in1, in2_mult=in2,
+                             mult=mult, shift=shift), executor)
