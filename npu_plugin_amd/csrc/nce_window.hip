@@ -17,7 +17,7 @@
 //     the per-channel bias.
 //   * the requantize runs in FP64 (see nce_ppe_device.h); shifts above 52 take the integer path.
 //   * MAXPOOL compares two channels per instruction (even / odd bytes as packed u16).
-#include "nce_ppe_device.h"
+#include "nce_conv_common.h"
 
 namespace nce {
 namespace {
@@ -65,13 +65,20 @@ struct WinArgs {
     uint32_t a_xor;   // 0x80808080 for i8 activations
     uint32_t fill;    // word of re-biased zero-point bytes for out-of-image taps
     int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
+    // I32 kernels (item count and tensor strides below 2^31): divisors of the item decomposition
+    int32_t nslab_full;            // channel groups of every slab but the last
+    FastDiv div_full, div_last;    // by the channel groups of a full slab / of the last slab
+    FastDiv div_bw, div_bh;
 };
 
 // KK = 2, 3, 5: KY == KX == KK known at compile time. All taps of an item are then requested before the first
 // one is used - unconditionally, from coordinates clamped into the image, with out-of-image taps replaced
 // afterwards - so that an item costs one memory round trip instead of one per tap. KK = 0: any window, taps
 // loaded one after the other.
-template <int MODE, int KK>
+// I32: the item count and every tensor stride fit 31 bits. The decomposition of an item into channel group, column,
+// row and image then runs on multiply-high divisions and index * stride is one 32 x 32 + 64 bit multiply-add;
+// the general kernel pays three 64-bit divisions per item, which cost more than the window itself.
+template <int MODE, int KK, bool I32>
 __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     // MODE_DW: [tap][SLAB_CH] floats of (w - zp_w); then per-channel FP64 scale constants
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -137,17 +144,32 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     for (int it = 0; it < a.items_per_thread; ++it) {
         const int64_t item = first + (int64_t)it * NT + threadIdx.x;
         if (item >= nitems) break;
-        const int32_t cg = (int32_t)(item % nslab);
-        int64_t r = item / nslab;
-        const int32_t bx = (int32_t)(r % box.bw);
-        r /= box.bw;
-        const int32_t by = (int32_t)(r % box.bh);
-        const int64_t n = r / box.bh;
+        int32_t cg, bx, by;
+        int64_t n;
+        if constexpr (I32) {
+            const uint32_t u = (uint32_t)item;
+            const uint32_t r1 = fdiv(u, nslab == a.nslab_full ? a.div_full : a.div_last);
+            cg = (int32_t)(u - r1 * (uint32_t)nslab);
+            const uint32_t r2 = fdiv(r1, a.div_bw);
+            bx = (int32_t)(r1 - r2 * (uint32_t)box.bw);
+            const uint32_t r3 = fdiv(r2, a.div_bh);
+            by = (int32_t)(r2 - r3 * (uint32_t)box.bh);
+            n = r3;
+        } else {
+            cg = (int32_t)(item % nslab);
+            int64_t r = item / nslab;
+            bx = (int32_t)(r % box.bw);
+            r /= box.bw;
+            by = (int32_t)(r % box.bh);
+            n = r / box.bh;
+        }
+        // index * stride
+        auto mul = [](int32_t i, int64_t stride) { return I32 ? (int64_t)i * (int32_t)stride : (int64_t)i * stride; };
         const int32_t oc = box.z0 + ((slab0 + cg) << 4);
         const int32_t oy = box.y0 + by, ox = box.x0 + bx;
         const int32_t iy0 = oy * t.sy - t.pt, ix0 = ox * t.sx - t.pl;
-        const uint8_t* src = t.in.data + n * t.in.sn + oc;
-        uint8_t* dst = t.out.data + n * t.out.sn + (int64_t)oy * t.out.sh + (int64_t)ox * t.out.sw + oc * t.out.sc;
+        const uint8_t* src = t.in.data + mul((int32_t)n, t.in.sn) + oc;
+        uint8_t* dst = t.out.data + mul((int32_t)n, t.out.sn) + mul(oy, t.out.sh) + mul(ox, t.out.sw) + oc * t.out.sc;
 
         if (MODE == MODE_MAX) {
             // even / odd bytes of each dword as packed u16; order-preserving re-bias for i8
@@ -159,7 +181,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
 #pragma unroll
                     for (int kx = 0; kx < KK; ++kx) {
                         const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
-                        v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                        v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                     }
 #pragma unroll
                 for (int ky = 0; ky < KK; ++ky)
@@ -183,7 +205,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 for (int kx = 0; kx < t.kx; ++kx) {
                     const int32_t ix = ix0 + kx;
                     if ((uint32_t)ix >= (uint32_t)t.in.w) continue;
-                    const uint4 va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                    const uint4 va = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                     const uint32_t wa[4] = {va.x ^ a.a_xor, va.y ^ a.a_xor, va.z ^ a.a_xor, va.w ^ a.a_xor};
 #pragma unroll
                     for (int d = 0; d < 4; ++d) {
@@ -234,7 +256,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
 #pragma unroll
                 for (int kx = 0; kx < KK; ++kx) {
                     const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
-                    v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                    v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                 }
 #pragma unroll
             for (int ky = 0; ky < KK; ++ky)
@@ -253,7 +275,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                     const int32_t ix = ix0 + kx;
                     uint4 va = make_uint4(a.fill, a.fill, a.fill, a.fill);
                     if (row_in && (uint32_t)ix < (uint32_t)t.in.w) {
-                        va = *reinterpret_cast<const uint4*>(src + (int64_t)iy * t.in.sh + (int64_t)ix * t.in.sw);
+                        va = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                         va.x ^= a.a_xor;
                         va.y ^= a.a_xor;
                         va.z ^= a.a_xor;
@@ -281,6 +303,14 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     }
 }
 
+template <int MODE, int KK, bool I32>
+hipError_t launch_window_i32(const WinArgs& a, int64_t blocks, int nslabs, size_t lds, hipStream_t s) {
+    static LdsGrant grant;  // large depthwise kernels: opt in to more than the default dynamic LDS
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE, KK, I32>), lds, 32 * 1024); e != hipSuccess) return e;
+    hipLaunchKernelGGL((window_kernel<MODE, KK, I32>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
+    return hipGetLastError();
+}
+
 template <int MODE, int KK>
 hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
     WinArgs a;
@@ -299,10 +329,16 @@ hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
     a.zpu = t.in.zp + (t.in.is_signed ? 128 : 0);
     a.fill = (uint32_t)a.zpu * 0x01010101u;
     const size_t lds = MODE == MODE_DW ? (size_t)t.ky * t.kx * SLAB_CH * sizeof(float) : 0;
-    static LdsGrant grant;  // large depthwise kernels: opt in to more than the default dynamic LDS
-    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE, KK>), lds, 32 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL((window_kernel<MODE, KK>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
-    return hipGetLastError();
+    const int32_t full = cgroups < SLAB_GROUPS ? cgroups : SLAB_GROUPS;
+    a.nslab_full = full;
+    a.div_full = make_fastdiv((uint32_t)full);
+    a.div_last = make_fastdiv((uint32_t)(cgroups - (nslabs - 1) * SLAB_GROUPS));
+    a.div_bw = make_fastdiv((uint32_t)box.bw);
+    a.div_bh = make_fastdiv((uint32_t)box.bh);
+    bool i32 = blocks * NT * a.items_per_thread < 0x7fffffffLL;
+    for (const int64_t st : {t.in.sn, t.in.sh, t.in.sw, t.out.sn, t.out.sh, t.out.sw}) i32 = i32 && st >= 0 && st <= 0x7fffffffLL;
+    if (i32) return launch_window_i32<MODE, KK, true>(a, blocks, nslabs, lds, s);
+    return launch_window_i32<MODE, KK, false>(a, blocks, nslabs, lds, s);
 }
 
 template <int MODE>
