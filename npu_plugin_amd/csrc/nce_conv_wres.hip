@@ -250,9 +250,13 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps the tile walk in scalar registers
     const int nwaves = blockDim.x >> 6;
     const int c16 = lane & 15;                  // pixel of a fragment this lane holds in matrix layout
+    // Pixel-major lane order: lane 4p + j carries 16-byte piece j ^ 2*(p >> 3) of pixel (or weight row) p. The four
+    // lanes of a pixel still cover its 64 bytes; the swap of the piece pairs for p >= 8 makes the 32 source lanes that
+    // each half of the wave reads in the permute distinct modulo 32 (without it they collide in pairs).
+    const int kswz = (lane & 3) ^ ((lane >> 4) & 2);
     const int pl = TRL ? lane >> 2 : c16;       // pixel and 16-byte piece this lane loads
-    const int kc = TRL ? lane & 3 : lane >> 4;
-    const int to_mfma = 4 * (4 * c16 + (lane >> 4));  // ds_bpermute source: lane 4p + k feeds lane 16k + p
+    const int kc = TRL ? kswz : lane >> 4;
+    const int to_mfma = 4 * (4 * c16 + ((lane >> 4) ^ (2 * (c16 >> 3))));  // ds_bpermute source of lane 16k + p: piece k of pixel p
 
     const int32_t oc0 = a.z0 + blockIdx.y * OCT;
     const int32_t noc = min(OCT, a.z0 + a.bc - oc0);
@@ -419,7 +423,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     // lanes), permutes the registers into operand order (lane 16k + i) and writes the fragment with one
     // linear, bank-conflict-free store.
     {
-        const int li = lane >> 2, lk = lane & 3;
+        const int li = lane >> 2, lk = kswz;
         const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
         // The last wave also derives the per-channel PPE constants (lane = channel) while its weight
         // loads are in flight.
