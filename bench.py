@@ -45,6 +45,19 @@ def make_workloads():
     }
 
 
+def make_scaled_workloads():
+    """The same layers at a batch that gives every CU several rounds of work: what the kernels reach once the
+    ~2.4 us launch gap and the per-workgroup set-up no longer dominate (the configurations above are 3-10 us long)."""
+    from npu_plugin_amd import workloads as W
+    return {
+        "cfg2_batch512": (lambda: W.cfg2(n=512), "mfma"),
+        "conv3x3_32x56x56x256_256": (lambda: W.conv_case(W.SEED + 20, 32, 56, 56, 256, 256, name="conv3x3_32x56x56x256_256"), "mfma"),
+        "cfg3_dw_batch128": (lambda: W.cfg3_dw(n=128), "hbm"),
+        "cfg3_maxpool_batch512": (lambda: W.cfg3_maxpool(n=512), "hbm"),
+        "cfg4_batch512": (lambda: W.cfg4(n=512), "hbm"),
+    }
+
+
 def time_task(ex, dc, steps, warmup):
     """Returns (wall seconds per step, event seconds per step)."""
     import torch
@@ -185,6 +198,7 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-others", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-scaled", action="store_true", help="skip the large-batch variants of the workloads")
     ap.add_argument("--per-layer", action="store_true", help="cfg5: print a per-task timing table on stderr")
     ap.add_argument("--traffic-reference", action="store_true",
                     help="also run plain 256 MiB device copies, the known-size reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
@@ -244,6 +258,12 @@ def main():
         if args.workload != "cfg5":
             others["cfg5"] = measure_graph(ex, max(5, args.steps // 10), max(2, args.warmup // 10))
         line["other_workloads"] = others
+        if not args.no_scaled:
+            scaled = {}
+            for name, (mk, bd) in make_scaled_workloads().items():
+                _, r = measure(ex, name, mk, bd, 20, 3)
+                scaled[name] = r
+            line["scaled_workloads"] = scaled
     ex.destroy()
     print(json.dumps(line))
 

@@ -29,6 +29,7 @@ constexpr int SLAB_CH = SLAB_GROUPS * 16;  // 128 channels
 constexpr int NT = 256;
 
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float ubyte_f32(uint32_t w, int i) {
     // the compiler turns this into v_cvt_f32_ubyte{i}
@@ -111,6 +112,20 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         }
         if (MODE == MODE_DW) {
             const uint8_t* row = t.weights + (int64_t)c * t.w_stride_oc;
+            if constexpr (KK > 0) {
+                // compile-time windows: (w - zp_w) of taps 2j and 2j + 1 as a pair of 16-bit values, the operand of
+                // v_dot2_i32_i16 (two taps of a channel per instruction)
+                uint32_t* s_w2 = reinterpret_cast<uint32_t*>(smem);
+                for (int j = 0; j < (KK * KK + 1) / 2; ++j) {
+                    int32_t wv[2] = {0, 0};
+                    for (int h = 0; h < 2; ++h) {
+                        const int tap = 2 * j + h;
+                        if (tap < KK * KK) wv[h] = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
+                    }
+                    wsum += wv[0] + wv[1];
+                    s_w2[j * SLAB_CH + ch] = ((uint32_t)wv[0] & 0xFFFFu) | ((uint32_t)wv[1] << 16);
+                }
+            } else
             for (int tap = 0; tap < ntaps; ++tap) {
                 const int32_t w = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
                 wsum += w;
@@ -258,15 +273,44 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                     const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
                     v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                 }
+            auto fixed = [&](int ky, int kx) {  // re-biased bytes of a tap, the zero point where it lies outside
+                const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+                const uint4 r = v[ky * KK + kx];
+                return make_uint4(ok ? r.x ^ a.a_xor : a.fill, ok ? r.y ^ a.a_xor : a.fill, ok ? r.z ^ a.a_xor : a.fill,
+                                  ok ? r.w ^ a.a_xor : a.fill);
+            };
+            if constexpr (MODE == MODE_DW) {
+                // Two taps per instruction: v_perm_b32 pairs byte i of both taps as 16-bit values, v_dot2_i32_i16
+                // multiplies the pair with the channel's weight pair and accumulates (exact, int32).
+                int32_t acci[16];
 #pragma unroll
-            for (int ky = 0; ky < KK; ++ky)
+                for (int i = 0; i < 16; ++i) acci[i] = 0;
+                const uint32_t* wp2 = reinterpret_cast<const uint32_t*>(smem) + (cg << 4);
 #pragma unroll
-                for (int kx = 0; kx < KK; ++kx) {
-                    const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
-                    const uint4 r = v[ky * KK + kx];
-                    tap(ky, kx, make_uint4(ok ? r.x ^ a.a_xor : a.fill, ok ? r.y ^ a.a_xor : a.fill, ok ? r.z ^ a.a_xor : a.fill,
-                                           ok ? r.w ^ a.a_xor : a.fill));
+                for (int j = 0; j < (KK * KK + 1) / 2; ++j) {
+                    const uint4 ra = fixed((2 * j) / KK, (2 * j) % KK);
+                    const uint4 rb = 2 * j + 1 < KK * KK ? fixed((2 * j + 1) / KK, (2 * j + 1) % KK) : make_uint4(0, 0, 0, 0);
+                    const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint4 w4 = *reinterpret_cast<const uint4*>(wp2 + j * SLAB_CH + 4 * d);
+                        const uint32_t wv[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t pair = __builtin_amdgcn_perm(wb[d], wa[d], 0x0c040c00u + (uint32_t)i * 0x00010001u);
+                            acci[4 * d + i] = __builtin_amdgcn_sdot2(__builtin_bit_cast(s16x2, pair), __builtin_bit_cast(s16x2, wv[i]),
+                                                                     acci[4 * d + i], false);
+                        }
+                    }
                 }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[i] = (float)acci[i];  // exact: below 2^24
+            } else {
+#pragma unroll
+                for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                    for (int kx = 0; kx < KK; ++kx) tap(ky, kx, fixed(ky, kx));
+            }
         } else {
             for (int ky = 0; ky < t.ky; ++ky) {
                 const int32_t iy = iy0 + ky;
