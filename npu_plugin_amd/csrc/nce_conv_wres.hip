@@ -759,6 +759,9 @@ hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t s
     if constexpr (BF < 4) {
         if (w.nsteps % 4 == 0) return launch_depth<NF, BF, 4>(w, mode, nwaves, tpw, stream);
         if (w.nsteps % 3 == 0) return launch_depth<NF, BF, 3>(w, mode, nwaves, tpw, stream);
+    } else {
+        // 64-pixel tiles: depth 3 only where depth 2 would need a padding step (9 steps: 3x3 over 64 channels)
+        if (w.nsteps % 2 != 0 && w.nsteps % 3 == 0) return launch_depth<NF, BF, 3>(w, mode, nwaves, tpw, stream);
     }
     return launch_depth<NF, BF, 2>(w, mode, nwaves, tpw, stream);
 }
