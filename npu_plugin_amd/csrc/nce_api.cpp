@@ -510,8 +510,26 @@ nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
     if (list == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
     if (list->ex->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
     if (hipSetDevice(list->ex->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
-    for (const Plan& p : list->plans) {
-        const nce_result_t r = launch_plan(list->ex, p, static_cast<hipStream_t>(hip_stream));
+    const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    for (size_t i = 0; i < list->plans.size(); ++i) {
+        const Plan& p = list->plans[i];
+        // A convolution directly followed by the residual add that consumes its output runs as one launch where the
+        // kernels allow it (both outputs are written; the bytes are those of the two tasks run one after the other).
+        if (p.task_type == NCE_TASK_CONV && p.boxes.size() == 1 && i + 1 < list->plans.size()) {
+            const Plan& q = list->plans[i + 1];
+            if (q.task_type == NCE_TASK_ELTWISE && q.boxes.size() == 1) {
+                const hipError_t e = nce::launch_conv_fused_add(p.dev, p.boxes[0], q.dev, q.boxes[0], stream);
+                if (e == hipSuccess) {
+                    ++i;
+                    continue;
+                }
+                if (e != hipErrorNotSupported) {
+                    list->ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
+                    return NCE_RESULT_ERROR_UNKNOWN;
+                }
+            }
+        }
+        const nce_result_t r = launch_plan(list->ex, p, stream);
         if (r != NCE_RESULT_SUCCESS) return r;
     }
     return NCE_RESULT_SUCCESS;

@@ -114,5 +114,12 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);
 hipError_t launch_pool(const TaskDev& t, const Box& box, bool is_max, hipStream_t stream);
 hipError_t launch_dwconv(const TaskDev& t, const Box& box, hipStream_t stream);
 hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream);
+// The convolution `conv` and the ELTWISE task `add` that directly follows it in a task list as ONE launch, when the add
+// reads the convolution's output and everything else allows it; hipErrorNotSupported (nothing launched) otherwise.
+hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& conv_box, const TaskDev& add, const Box& add_box, hipStream_t stream);
+struct FuseAdd;
+// Integer constants of a uniform-scale ELTWISE add whose first input is `first_is_other ? other : produced`; false when
+// the task needs another arithmetic path.
+bool eltwise_fuse_params(const TaskDev& add, bool produced_is_in1, FuseAdd* out);
 
 }  // namespace nce

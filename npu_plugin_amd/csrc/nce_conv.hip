@@ -234,8 +234,8 @@ hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
-    ConvArgs a;
+// Launch arguments of a convolution over one box; hipSuccess, or the error to return.
+static hipError_t make_conv_args(const TaskDev& t, const Box& box, ConvArgs& a) {
     a.in = t.in.data;
     a.in_sn = t.in.sn;
     a.in_sh = t.in.sh;
@@ -285,6 +285,60 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     a.pitchpx = t.in.w + t.pl + t.pr;
     a.nslots_max = a.rows_max = a.nchunks = a.halo_bytes = 0;
     a.ppe = t.ppe;
+    return hipSuccess;
+}
+
+static bool same_dense_tensor(const TensorDev& x, const TensorDev& y) {
+    return x.data == y.data && x.n == y.n && x.h == y.h && x.w == y.w && x.c == y.c && x.sc == 1 && y.sc == 1 && x.sw == y.sw &&
+           x.sh == y.sh && x.sn == y.sn && x.sw == x.c && x.sh == (int64_t)x.w * x.c && x.sn == (int64_t)x.h * x.sh;
+}
+static bool same_shape_dense(const TensorDev& x, const TensorDev& like) {
+    return x.n == like.n && x.h == like.h && x.w == like.w && x.c == like.c && x.sc == 1 && x.sw == x.c &&
+           x.sh == (int64_t)x.w * x.c && x.sn == (int64_t)x.h * x.sh;
+}
+static bool overlaps(const TensorDev& x, const TensorDev& y) {
+    const uint8_t* xe = x.data + (int64_t)x.n * x.sn;
+    const uint8_t* ye = y.data + (int64_t)y.n * y.sn;
+    return x.data < ye && y.data < xe;
+}
+
+hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskDev& add, const Box& ab, hipStream_t stream) {
+    if (getenv("NCE_HIP_NO_FUSE") || getenv("NCE_HIP_CONV_PATH")) return hipErrorNotSupported;
+    const TensorDev& o = conv.out;
+    const bool conv_full = cb.x0 == 0 && cb.y0 == 0 && cb.z0 == 0 && cb.bw == o.w && cb.bh == o.h && cb.bc == o.c;
+    const bool add_full = ab.x0 == 0 && ab.y0 == 0 && ab.z0 == 0 && ab.bw == add.out.w && ab.bh == add.out.h && ab.bc == add.out.c;
+    if (!conv_full || !add_full || add.table != nullptr) return hipErrorNotSupported;
+    const bool is_in1 = same_dense_tensor(add.in, o), is_in2 = same_dense_tensor(add.in2, o);
+    if (is_in1 == is_in2) return hipErrorNotSupported;  // neither input, or both
+    const TensorDev& other = is_in1 ? add.in2 : add.in;
+    // The add must see the convolution's stored type; its other input and its output have the same dense shape and
+    // do not touch the convolution's output (the output may be the other input: each element is read before it is written,
+    // by the same lane).
+    if ((is_in1 ? add.in : add.in2).is_signed != o.is_signed) return hipErrorNotSupported;
+    if (!same_shape_dense(other, o) || !same_shape_dense(add.out, o) || overlaps(other, o) || overlaps(add.out, o)) return hipErrorNotSupported;
+    if (overlaps(add.out, other) && add.out.data != other.data) return hipErrorNotSupported;
+    // ... nor the convolution's operands
+    if (overlaps(add.out, conv.in)) return hipErrorNotSupported;
+    const uint8_t* const ob = add.out.data;
+    const uint8_t* const oe = ob + (int64_t)add.out.n * add.out.sn;
+    const uint8_t* const wb = conv.weights;
+    const uint8_t* const we = wb + (int64_t)o.c * conv.w_stride_oc;
+    const uint8_t* const tb = reinterpret_cast<const uint8_t*>(conv.table);
+    const uint8_t* const te = tb + (int64_t)o.c * conv.table_stride * 4;
+    if ((ob < we && wb < oe) || (ob < te && tb < oe)) return hipErrorNotSupported;
+    FuseAdd fz;
+    if (!eltwise_fuse_params(add, is_in1, &fz)) return hipErrorNotSupported;
+    fz.other = other.data;
+    fz.out = add.out.data;
+    ConvArgs a;
+    if (const hipError_t e = make_conv_args(conv, cb, a); e != hipSuccess) return e;
+    if (a.M == 0 || cb.bc == 0) return hipErrorNotSupported;
+    return launch_conv_wres(a, stream, false, &fz);
+}
+
+hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
+    ConvArgs a;
+    if (const hipError_t e0 = make_conv_args(t, box, a); e0 != hipSuccess) return e0;
     if (a.M == 0 || box.bc == 0) return hipSuccess;
     // tuning and test knob: 1 = skip the weights-resident kernel, 2 = gather kernel only
     const char* path_env = getenv("NCE_HIP_CONV_PATH");

@@ -195,6 +195,23 @@ hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream);
 // Returns hipErrorNotSupported when the shape does not fit the halo kernel (caller falls back).
 hipError_t launch_conv_halo(const ConvArgs& a, hipStream_t stream);
 // allow_chunked: also take reductions longer than one LDS slice (weights staged chunk by chunk)
-hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked);
+// A residual add fused into the epilogue of the convolution that produces one of its inputs (task lists: a
+// convolution directly followed by an ELTWISE task reading its output). The convolution's own output is still
+// written; the add's output is computed from the stored bytes, so both tensors hold what the two tasks give.
+// All three tensors of the add are dense NHWC of the convolution's output shape: element offsets coincide.
+struct FuseAdd {
+    const uint8_t* other;  // the add's other input
+    uint8_t* out;          // the add's output
+    uint32_t mults;        // input multiplier of the convolution's value | of the other input << 16
+    uint32_t in_flip;      // 0x80808080 for signed inputs (they enter the 16-bit dot product 128 higher)
+    int32_t c0h;           // -(mults . zero points), less 128 * (sum of multipliers) for signed inputs
+    int32_t mq;            // quant_mult * 2^(32 - shift)
+    int64_t cq;            // (2^(shift-1) + zero point * 2^shift) * 2^(32 - shift)
+    int32_t ilo, ihi;      // clamp bounds (signed outputs 128 higher)
+    uint32_t flip;         // 0x80808080 for signed outputs
+};
+
+// fuse: optional; hipErrorNotSupported when the kernel variant that would run the task cannot carry the add.
+hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse = nullptr);
 
 }  // namespace nce

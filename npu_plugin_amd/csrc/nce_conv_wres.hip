@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 
 namespace nce {
 
@@ -46,6 +47,8 @@ struct WresArgs {
     // The tensor strides once more as 32-bit values (the host checks that they fit): index * stride is then one
     // 32 x 32 + 64 bit multiply-add instead of a 64-bit multiplication.
     int32_t in_sn32, in_sh32, in_sw32, out_sn32, out_sh32, out_sw32;
+    FuseAdd fz;         // kernels with LM_PLAIN_FZ only
+    int32_t fused;      // host: the launch must carry the add in fz (or fail with hipErrorNotSupported)
 };
 
 // This file is compiled twice (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
@@ -121,13 +124,16 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
     return e;
 }
 
-template <int NF, int BF, int PMODE>
+typedef unsigned short fz_u16x2 __attribute__((ext_vector_type(2)));
+
+template <int NF, int BF, int PMODE, bool FZ = false>
 __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
                                               const v4i (&acc)[NF][BF], const int32_t (&dws)[BF], int q, int noc,
                                               uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
-                                              const EpiPack& ep) {
+                                              const EpiPack& ep, const FuseAdd* fz = nullptr, const uint4* other = nullptr) {
     const int ch0 = 4 * NF * q;
     if (ch0 >= noc) return;
+    static_assert(!FZ || NF == 4, "fused add: a lane holds 16 channels");
     uint32_t wo[BF][NF];
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
@@ -201,6 +207,31 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
         if constexpr (NF == 4) store_channels16(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
         else store_channels8(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1]);
     }
+    if constexpr (FZ) {
+        // The add on the bytes just stored (a.out_sc == 1 here): byte i of both inputs as a pair of 16-bit values, one
+        // 16-bit dot product with the two input multipliers, the high word of one multiply-add, clamp, byte insert.
+#pragma unroll
+        for (int x = 0; x < BF; ++x) {
+            if (!valid[x]) continue;
+            const uint32_t ob[4] = {other[x].x, other[x].y, other[x].z, other[x].w};
+            uint32_t r[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t ua = wo[x][d] ^ fz->in_flip, ub = ob[d] ^ fz->in_flip;
+                uint32_t packed = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t pair = __builtin_amdgcn_perm(ub, ua, 0x0c040c00u + (uint32_t)i * 0x00010001u);
+                    const int32_t sum = (int32_t)__builtin_amdgcn_udot2(__builtin_bit_cast(fz_u16x2, pair), __builtin_bit_cast(fz_u16x2, fz->mults),
+                                                                         (uint32_t)fz->c0h, false);
+                    const int32_t y = clamp_med3((int32_t)(((int64_t)sum * fz->mq + fz->cq) >> 32), fz->ilo, fz->ihi);
+                    packed = i == 0 ? (uint32_t)y : (packed | ((uint32_t)y << (8 * i)));
+                }
+                r[d] = packed ^ fz->flip;
+            }
+            *reinterpret_cast<uint4*>(fz->out + ((dst[x] + ch0) - a.out)) = make_uint4(r[0], r[1], r[2], r[3]);
+        }
+    }
 }
 
 // D: reduction steps whose activation loads are in flight per wave; the host picks a D that divides the step
@@ -218,12 +249,13 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
 // instruction per step and pixel fragment against an all-ones operand, every row of the result is the sum),
 // the constant joins the per-channel constants.
 // LM packs the three flags: 0 plain, 1 TRL, 2 TBL, 3 plain + ASUM, 4 TRL + ASUM.
-enum { LM_PLAIN = 0, LM_TRL = 1, LM_TBL = 2, LM_PLAIN_ASUM = 3, LM_TRL_ASUM = 4 };
+enum { LM_PLAIN = 0, LM_TRL = 1, LM_TBL = 2, LM_PLAIN_ASUM = 3, LM_TRL_ASUM = 4, LM_PLAIN_FZ = 5 };  // 5: plain + fused residual add
 template <int NF, int BF, int MODE, int D, int LM>
 __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     constexpr bool TRL = LM == LM_TRL || LM == LM_TRL_ASUM;
     constexpr bool TBL = LM == LM_TBL;
     constexpr bool ASUM = LM == LM_PLAIN_ASUM || LM == LM_TRL_ASUM;
+    constexpr bool FZ = LM == LM_PLAIN_FZ;
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
     constexpr int WB = 4;      // weight loads in flight per lane while staging
@@ -598,6 +630,15 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         for (int f = 0; f < NF; ++f)
 #pragma unroll
             for (int x = 0; x < BF; ++x) acc[f][x] = v4i{0, 0, 0, 0};
+        // Fused residual add: the other input's 16 channels of each of the lane's pixels are requested now and travel
+        // while the reduction runs (unconditionally: a lane without a pixel or past the slice's last channel reads a
+        // duplicate address inside the tensor).
+        uint4 other[FZ ? BF : 1];
+        if constexpr (FZ) {
+            const int ch0 = min(16 * (lane >> 4), noc - 16);
+#pragma unroll
+            for (int x = 0; x < BF; ++x) other[x] = *reinterpret_cast<const uint4*>(w.fz.other + ((dst[x] + ch0) - a.out));
+        }
         // Steady state: every step consumes one ring slot and refills it for step + D, with no branch
         // around the load, so that the wait before a step covers exactly the loads older than its own.
         v4i asum[BF];
@@ -671,11 +712,11 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         int32_t dws[BF];  // every row of asum holds the pixel's sum: register 0 of this lane is its column's
 #pragma unroll
         for (int x = 0; x < BF; ++x) dws[x] = ASUM ? a.dw * asum[x][0] : 0;
-        if (pmode == PPE_MODE_HI) wres_epilogue<NF, BF, PPE_MODE_HI>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_HI_SLOPE) wres_epilogue<NF, BF, PPE_MODE_HI_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
-        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
-        else wres_epilogue<NF, BF, PPE_MODE_INT>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep);
+        if (pmode == PPE_MODE_HI) wres_epilogue<NF, BF, PPE_MODE_HI, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
+        else if (pmode == PPE_MODE_HI_SLOPE) wres_epilogue<NF, BF, PPE_MODE_HI_SLOPE, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
+        else if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
+        else if (pmode == PPE_MODE_SLOPE) wres_epilogue<NF, BF, PPE_MODE_SLOPE, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
+        else wres_epilogue<NF, BF, PPE_MODE_INT, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
         t += nwaves;
         if (t < t_end) {
             setup();
@@ -711,6 +752,14 @@ hipError_t launch_depth(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t 
     // Transposed loads: measured to pay for every kernel larger than 1x1 and for long 1x1 reductions, once
     // pixels are more than 64 bytes apart (the per-lane mode serves channel counts below that).
     const bool trl = D >= 2 && mode != WRES_GENERIC && w.a.in_sw > 64 && (w.ntaps > 1 || w.nsteps >= 32);
+    if (w.fused) {
+        // The fused residual add exists for the 64-channel kernels with plain loads and every tap inside the image
+        // (the 1x1 convolutions that close a residual block).
+        if constexpr (NF == 4) {
+            if (mode == WRES_FAST && !trl && w.a.dw == 0 && w.a.out_sc == 1) return launch_one<NF, BF, WRES_FAST, D, LM_PLAIN_FZ>(w, nwaves, tpw, stream);
+        }
+        return hipErrorNotSupported;
+    }
     if constexpr (D == 1 || D == 2 || D == 4) {
         if (w.a.dw != 0) {  // activation sums for the weight zero-point term
             if constexpr (D >= 2) {
@@ -1109,12 +1158,15 @@ hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, h
     return launch_bf<4>(w, bf, mode, nwaves, tpw, stream);
 }
 #else
-hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked) {
+hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse) {
     if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
     if (a.M > 0x7fffffff - 64 * 1024) return hipErrorNotSupported;
     WresArgs w;
     w.a = a;
+    w.fused = fuse != nullptr;
+    if (fuse) w.fz = *fuse;
+    else memset(&w.fz, 0, sizeof(w.fz));
     w.k16 = a.KG;
     w.nsteps = (a.KG + 3) / 4;
     w.nc64 = a.IC / 64;
@@ -1132,7 +1184,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     w.out_sh32 = (int32_t)a.out_sh;
     w.out_sw32 = (int32_t)a.out_sw;
     const size_t wl4 = (size_t)((w.nsteps + 1) / 2 * 2) * 4 * 1024, wl2 = wl4 / 2;  // with the padding step
-    if (wl2 > kWresLdsCap) return allow_chunked ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
+    if (wl2 > kWresLdsCap) return allow_chunked && !w.fused ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
 
     // every tap of every output pixel of the box inside the image?
     const int64_t iy_lo = (int64_t)a.y0 * a.SY - a.PT, iy_hi = (int64_t)(a.y0 + a.bh - 1) * a.SY - a.PT + a.KY - 1;
@@ -1143,7 +1195,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
                a.bw == a.W && a.bh == a.H && a.in_sh == (int64_t)a.W * a.in_sw && a.in_sn == (int64_t)a.H * a.in_sh &&
                a.out_sh == (int64_t)a.bw * a.out_sw && a.out_sn == (int64_t)a.bh * a.out_sh;
     // one bit per tap, bit 31 stays clear; larger kernels take the chunked kernel's row / column bits
-    if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return allow_chunked ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
+    if (mode == WRES_FAST_MASK && a.KY * a.KX > 31) return allow_chunked && !w.fused ? launch_conv_wres_chunked(w, stream) : hipErrorNotSupported;
 
     // Shape of the work: nf channel fragments per slice, bf pixel fragments per wave tile. Measured on
     // MI355X over the ResNet-50 layer shapes, the best shape is always the LARGEST tile that still
@@ -1181,6 +1233,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
             if (ftpw >= 1) tpw = ftpw, forced_tpw = true;  // (0: keep the automatic choice below)
         }
     }
+    if (w.fused && nf4_ok) nf = 4;  // (the fused add exists for the 64-channel kernels)
     w.tpg = forced_tpw ? 0 : pick_tpg(nf, bf, nw);
     if (nf == 4) return launch_wres_nf4(w, bf, mode, nw, tpw, stream);
     return launch_bf<2>(w, bf, mode, nw, tpw, stream);

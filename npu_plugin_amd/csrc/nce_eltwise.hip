@@ -6,7 +6,7 @@
 // (global_load_dwordx4 x2, global_store_dwordx4 x1), 48 algorithmic bytes per 16 outputs. The
 // requantize runs in FP64 (exact, see nce_ppe_device.h); per-channel tables and shifts above 52
 // take the integer path.
-#include "nce_ppe_device.h"
+#include "nce_conv_common.h"
 
 namespace nce {
 namespace {
@@ -137,17 +137,10 @@ void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
     else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
 
-}  // namespace
 
-hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) {
-    EltArgs a;
+// Fills the launch arguments and returns the arithmetic path (a PPE_MODE_* value, PATH_TABLE or PATH_HI).
+static int prepare(const TaskDev& t, EltArgs& a) {
     a.t = t;
-    a.box = box;
-    a.nchunks = (int64_t)t.out.n * box.bh * box.bw * (box.bc >> 4);
-    if (a.nchunks == 0) return hipSuccess;
-    const bool full = box.x0 == 0 && box.y0 == 0 && box.z0 == 0 && box.bw == t.out.w && box.bh == t.out.h &&
-                      box.bc == t.out.c;
-    const bool flat = full && is_dense_nhwc(t.in) && is_dense_nhwc(t.in2) && is_dense_nhwc(t.out);
     a.c0 = -(t.ppe.in1_mult * t.in.zp + t.ppe.in2_mult * t.in2.zp);
     const int shift = t.ppe.quant_shift;
     a.M = ldexp((double)t.ppe.quant_mult, -shift);
@@ -186,6 +179,34 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
             a.c0h = a.c0 - (t.in.is_signed ? 128 * (t.ppe.in1_mult + t.ppe.in2_mult) : 0);
         }
     }
+    return path;
+}
+
+}  // namespace
+
+bool eltwise_fuse_params(const TaskDev& add, bool produced_is_in1, FuseAdd* out) {
+    EltArgs a;
+    if (prepare(add, a) != PATH_HI || add.in.is_signed != add.in2.is_signed) return false;
+    out->mults = produced_is_in1 ? a.mults : ((a.mults >> 16) | (a.mults << 16));
+    out->in_flip = a.in_flip;
+    out->c0h = a.c0h;
+    out->mq = a.mq;
+    out->cq = a.cq;
+    out->ilo = a.ilo;
+    out->ihi = a.ihi;
+    out->flip = a.flip;
+    return true;
+}
+
+hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) {
+    EltArgs a;
+    a.box = box;
+    a.nchunks = (int64_t)t.out.n * box.bh * box.bw * (box.bc >> 4);
+    if (a.nchunks == 0) return hipSuccess;
+    const bool full = box.x0 == 0 && box.y0 == 0 && box.z0 == 0 && box.bw == t.out.w && box.bh == t.out.h &&
+                      box.bc == t.out.c;
+    const bool flat = full && is_dense_nhwc(t.in) && is_dense_nhwc(t.in2) && is_dense_nhwc(t.out);
+    const int path = prepare(t, a);
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (flat) launch_path<true>(a, path, (int)blocks, stream);

@@ -661,3 +661,67 @@ def test_eltwise_integer_path_boundaries(executor, signed, shift, mult):
         zp = -5 if signed else 128
         check(K.eltwise_case(5000 + shift, 2, 5, 7, 48, signed=signed, zp_a=zp, zp_b=zp + 3, out_zp=zp, in1_mult=in1, in2_mult=in2,
                              mult=mult, shift=shift), executor)
+
+
+def _conv_then_add(executor, monkeypatch, conv_kw, add_kw, conv_first, in_place, config="4,2,8,0", fuse=True):
+    """A convolution directly followed by the add that reads its output, through one task list; returns the two
+    outputs from the GPU and from the oracle."""
+    import torch
+    if config:
+        monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    if not fuse:
+        monkeypatch.setenv("NCE_HIP_NO_FUSE", "1")
+    c1 = K.conv_case(**conv_kw)
+    y1 = K.run_oracle(c1)
+    n, h, w, c = c1.out_shape
+    c2 = K.eltwise_case(7001, n, h, w, c, signed=c1.out_signed, **add_kw)
+    if conv_first:
+        c2.input = y1
+    else:
+        c2.weights = y1
+    y2 = K.run_oracle(c2)
+    d1 = K.DeviceCase(c1)
+    d2 = K.DeviceCase(c2)
+    other = d2.weights if conv_first else d2.input
+    out2 = other if in_place else d2.output
+    t2 = K.build_task(c2, d1.output if conv_first else other, other if conv_first else d1.output, None, out2)
+    tl = executor.task_list()
+    tl.append(d1.task)
+    tl.append(t2)
+    stream = torch.cuda.current_stream().cuda_stream
+    tl.enqueue(stream)
+    executor.synchronize(stream)
+    tl.destroy()
+    return d1.output.cpu().numpy(), out2.cpu().numpy(), y1, y2
+
+
+@pytest.mark.parametrize("conv_first,in_place", [(True, False), (False, False), (True, True), (False, True)])
+@pytest.mark.parametrize("config", ["4,4,8,0", "4,2,8,0", "4,1,8,0", "2,2,8,0", None])
+def test_conv_with_fused_residual_add(executor, monkeypatch, conv_first, in_place, config):
+    # 1x1 convolutions that close a residual block, followed by the block's add: one launch for both on the 64-channel
+    # kernels (a 32-channel configuration and the automatic choice fall back to two launches where they must).
+    for ic, oc, out_signed, out_zp in ((64, 256, False, 128), (128, 80, True, -3), (256, 64, False, 0), (512, 128, False, 7)):
+        lo, hi = (-128, 127) if out_signed else (0, 255)
+        conv_kw = dict(seed=7100 + ic, n=2, h=9, w=11, ic=ic, oc=oc, k=(1, 1), pads=(0, 0, 0, 0), out_signed=out_signed, out_zp=out_zp,
+                       ppe=dict(mode=nce.PPE_NOOP, clamp_low=lo + 5, clamp_high=hi))
+        add_kw = dict(zp_a=out_zp, zp_b=(out_zp + 9) if not out_signed else -20, out_zp=out_zp, in1_mult=20971, in2_mult=31457,
+                      mult=25600, shift=30)
+        g1, g2, y1, y2 = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, conv_first, in_place, config)
+        assert np.array_equal(g1, y1), "convolution output"
+        assert np.array_equal(g2, y2), "add output"
+
+
+def test_conv_fused_add_equals_two_launches(executor, monkeypatch):
+    # the same pair with the fusion switched off, and pairs the fusion must refuse (a 3x3 with padding, an add with a slope)
+    conv_kw = dict(seed=7200, n=1, h=14, w=14, ic=128, oc=192, k=(1, 1), pads=(0, 0, 0, 0))
+    add_kw = dict(zp_a=128, zp_b=100, out_zp=120)
+    a = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, True, False, "4,2,8,0", fuse=True)
+    b = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, True, False, "4,2,8,0", fuse=False)
+    for x, y in zip(a, b):
+        assert np.array_equal(x, y)
+    monkeypatch.delenv("NCE_HIP_NO_FUSE")
+    for conv_kw2, add_kw2 in ((dict(conv_kw, k=(3, 3), pads=(1, 1, 1, 1)), add_kw),
+                              (conv_kw, dict(add_kw, ppe_extra=dict(mode=nce.PPE_LPRELU, lrelu_mult=1638, lrelu_shift=14))),
+                              (conv_kw, dict(add_kw, shift=40))):
+        g1, g2, y1, y2 = _conv_then_add(executor, monkeypatch, conv_kw2, add_kw2, False, False, "4,2,8,0")
+        assert np.array_equal(g1, y1) and np.array_equal(g2, y2)
