@@ -155,7 +155,7 @@ def measure_graph(ex, steps, warmup, batch=32, per_layer=False):
     other_bytes = sum(graph.layer_bytes(L) for L in graph.layers if L.task_type != 0)
     roof = {"bound": "mfma", "achieved": ops / ev / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
             "frac": ops / ev / 1e12 / PEAK_INT8_TOPS, "traffic": None, "kernel_us": ev * 1e6,
-            "note": "whole graph per step: 53 conv kernels + 1 max pool + 16 adds, launched back to back"}
+            "note": "whole graph per step: 53 conv + 1 max pool + 16 add tasks from one task list, launched back to back; an add that directly follows the convolution producing its input runs inside that convolution's launch"}
     layers = per_layer_table(ex, dg) if per_layer else None
     if layers:
         for r in layers:
