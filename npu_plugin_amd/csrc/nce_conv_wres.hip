@@ -51,8 +51,9 @@ struct WresArgs {
     int32_t fused;      // host: the launch must carry the add in fz (or fail with hipErrorNotSupported)
 };
 
-// This file is compiled twice (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
-// the 32-channel kernels and the chunked kernel, WRES_PART 1 the 64-channel kernels behind this entry point.
+// This file is compiled three times (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
+// the 32-channel kernels and the chunked kernel, WRES_PART 1 the 64-channel kernels with 16- and 32-pixel tiles behind this
+// entry point, WRES_PART 2 those with 64-pixel tiles.
 #ifndef WRES_PART
 #define WRES_PART 0
 #endif
@@ -1154,8 +1155,15 @@ hipError_t launch_bf(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStre
 }  // namespace
 
 #if WRES_PART == 1
+hipError_t launch_wres_nf4_bf4(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream);
 hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream) {
-    return launch_bf<4>(w, bf, mode, nwaves, tpw, stream);
+    if (bf == 4) return launch_wres_nf4_bf4(w, mode, nwaves, tpw, stream);
+    if (bf == 2) return launch_mode<4, 2>(w, mode, nwaves, tpw, stream);
+    return launch_mode<4, 1>(w, mode, nwaves, tpw, stream);
+}
+#elif WRES_PART == 2
+hipError_t launch_wres_nf4_bf4(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
+    return launch_mode<4, 4>(w, mode, nwaves, tpw, stream);
 }
 #else
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse) {
