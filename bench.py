@@ -179,7 +179,7 @@ def cpu_baseline(case, bound, budget_s=12.0):
         run_oracle(case, cores)
         n += 1
         dt = time.perf_counter() - t0
-        if dt > budget_s or n >= 50:
+        if dt > budget_s or n >= 100:
             break
     per = dt / n
     if bound == "mfma":
