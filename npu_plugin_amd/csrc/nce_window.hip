@@ -202,11 +202,11 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 for (int ky = 0; ky < KK; ++ky)
 #pragma unroll
                     for (int kx = 0; kx < KK; ++kx) {
-                        const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+                        // (An out-of-image tap was loaded from its coordinates clamped into the image. Every window
+                        // reaches into the image - the host sends other tasks to the general kernel -, so the clamped
+                        // pixel is one of the window's own in-image pixels and the maximum is unchanged.)
                         const uint4 va = v[ky * KK + kx];
-                        // (an out-of-image tap becomes 0, the smallest re-biased value: it never wins)
-                        const uint32_t wa[4] = {ok ? va.x ^ a.a_xor : 0u, ok ? va.y ^ a.a_xor : 0u, ok ? va.z ^ a.a_xor : 0u,
-                                                ok ? va.w ^ a.a_xor : 0u};
+                        const uint32_t wa[4] = {va.x ^ a.a_xor, va.y ^ a.a_xor, va.z ^ a.a_xor, va.w ^ a.a_xor};
 #pragma unroll
                         for (int d = 0; d < 4; ++d) {
                             me[d] = pk_max_u16(me[d], wa[d] & 0x00FF00FFu);
@@ -387,6 +387,12 @@ hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
 
 template <int MODE>
 hipError_t launch_window(const TaskDev& t, const Box& box, hipStream_t s) {
+    if (MODE == MODE_MAX) {
+        // the compile-time windows of the max pool rely on every window of the box overlapping the image
+        const bool reach = t.pt < t.ky && t.pl < t.kx && (int64_t)(box.y0 + box.bh - 1) * t.sy - t.pt <= t.in.h - 1 &&
+                           (int64_t)(box.x0 + box.bw - 1) * t.sx - t.pl <= t.in.w - 1;
+        if (!reach) return launch_window_kk<MODE, 0>(t, box, s);
+    }
     if (t.ky == 3 && t.kx == 3) return launch_window_kk<MODE, 3>(t, box, s);
     if (t.ky == 2 && t.kx == 2) return launch_window_kk<MODE, 2>(t, box, s);
     if (t.ky == 5 && t.kx == 5) return launch_window_kk<MODE, 5>(t, box, s);
