@@ -10,11 +10,13 @@
 // Memory-bound kernels: a lane owns one 16-channel group (one 128-bit load per tap) of one output
 // pixel; adjacent lanes own adjacent channel groups, so a wavefront reads whole NHWC pixels
 // contiguously. Arithmetic is kept below the memory time:
-//   * sums run in FP32 on v_cvt_f32_ubyteN (byte -> float in one instruction) + v_fma_f32. Every
-//     partial sum is an integer below 2^24 (121 taps * 255 * 255), so FP32 is exact.
+//   * depthwise sums over a compile-time window (2x2, 3x3, 5x5) take two taps per instruction: v_perm_b32
+//     pairs a byte of two taps as 16-bit values, v_dot2_i32_i16 multiplies them with the channel's weight
+//     pair. Other sums run in FP32 on v_cvt_f32_ubyteN (byte -> float in one instruction) + v_fma_f32:
+//     every partial sum is an integer below 2^24 (121 taps * 255 * 255), so FP32 is exact.
 //   * bytes are taken as unsigned (i8 storage is re-biased by x ^ 0x80) and out-of-image taps are
 //     filled with the zero point, so they contribute 0; the constant  -zp * sum(w)  is folded into
-//     the per-channel bias.
+//     the per-channel bias. (Max pool keeps the clamped in-window pixel instead: the maximum is the same.)
 //   * the requantize runs in FP64 (see nce_ppe_device.h); shifts above 52 take the integer path.
 //   * MAXPOOL compares two channels per instruction (even / odd bytes as packed u16).
 #include "nce_conv_common.h"
@@ -273,11 +275,23 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                     const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
                     v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                 }
-            auto fixed = [&](int ky, int kx) {  // re-biased bytes of a tap, the zero point where it lies outside
-                const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+            // Out-of-image taps take the zero point. Most wavefronts hold no such tap: the replacement runs only where
+            // one does (uniform branch), the re-biasing XOR always.
+            const bool inside = iy0 >= 0 && ix0 >= 0 && iy0 + KK <= t.in.h && ix0 + KK <= t.in.w;
+            if (!__all(inside)) {
+                const uint32_t fr = a.fill ^ a.a_xor;
+#pragma unroll
+                for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                    for (int kx = 0; kx < KK; ++kx) {
+                        const bool ok = (uint32_t)(iy0 + ky) < (uint32_t)t.in.h && (uint32_t)(ix0 + kx) < (uint32_t)t.in.w;
+                        uint4& r = v[ky * KK + kx];
+                        r = make_uint4(ok ? r.x : fr, ok ? r.y : fr, ok ? r.z : fr, ok ? r.w : fr);
+                    }
+            }
+            auto fixed = [&](int ky, int kx) {  // re-biased bytes of a tap
                 const uint4 r = v[ky * KK + kx];
-                return make_uint4(ok ? r.x ^ a.a_xor : a.fill, ok ? r.y ^ a.a_xor : a.fill, ok ? r.z ^ a.a_xor : a.fill,
-                                  ok ? r.w ^ a.a_xor : a.fill);
+                return make_uint4(r.x ^ a.a_xor, r.y ^ a.a_xor, r.z ^ a.a_xor, r.w ^ a.a_xor);
             };
             if constexpr (MODE == MODE_DW) {
                 // Two taps per instruction: v_perm_b32 pairs byte i of both taps as 16-bit values, v_dot2_i32_i16
