@@ -200,6 +200,10 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                         const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
                         v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                     }
+                if (a.a_xor != 0) {  // uniform: only i8 storage needs the order-preserving re-bias
+#pragma unroll
+                    for (int i = 0; i < KK * KK; ++i) v[i] = make_uint4(v[i].x ^ a.a_xor, v[i].y ^ a.a_xor, v[i].z ^ a.a_xor, v[i].w ^ a.a_xor);
+                }
 #pragma unroll
                 for (int ky = 0; ky < KK; ++ky)
 #pragma unroll
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                         // reaches into the image - the host sends other tasks to the general kernel -, so the clamped
                         // pixel is one of the window's own in-image pixels and the maximum is unchanged.)
                         const uint4 va = v[ky * KK + kx];
-                        const uint32_t wa[4] = {va.x ^ a.a_xor, va.y ^ a.a_xor, va.z ^ a.a_xor, va.w ^ a.a_xor};
+                        const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
 #pragma unroll
                         for (int d = 0; d < 4; ++d) {
                             me[d] = pk_max_u16(me[d], wa[d] & 0x00FF00FFu);
@@ -276,10 +280,14 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                     v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
                 }
             // Out-of-image taps take the zero point. Most wavefronts hold no such tap: the replacement runs only where
-            // one does (uniform branch), the re-biasing XOR always.
+            // one does (uniform branch).
             const bool inside = iy0 >= 0 && ix0 >= 0 && iy0 + KK <= t.in.h && ix0 + KK <= t.in.w;
+            if (a.a_xor != 0) {  // uniform: i8 storage is re-biased to unsigned bytes
+#pragma unroll
+                for (int i = 0; i < KK * KK; ++i) v[i] = make_uint4(v[i].x ^ a.a_xor, v[i].y ^ a.a_xor, v[i].z ^ a.a_xor, v[i].w ^ a.a_xor);
+            }
             if (!__all(inside)) {
-                const uint32_t fr = a.fill ^ a.a_xor;
+                const uint32_t fr = a.fill;
 #pragma unroll
                 for (int ky = 0; ky < KK; ++ky)
 #pragma unroll
@@ -289,10 +297,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                         r = make_uint4(ok ? r.x : fr, ok ? r.y : fr, ok ? r.z : fr, ok ? r.w : fr);
                     }
             }
-            auto fixed = [&](int ky, int kx) {  // re-biased bytes of a tap
-                const uint4 r = v[ky * KK + kx];
-                return make_uint4(r.x ^ a.a_xor, r.y ^ a.a_xor, r.z ^ a.a_xor, r.w ^ a.a_xor);
-            };
+            auto fixed = [&](int ky, int kx) { return v[ky * KK + kx]; };  // re-biased bytes of a tap
             if constexpr (MODE == MODE_DW) {
                 // Two taps per instruction: v_perm_b32 pairs byte i of both taps as 16-bit values, v_dot2_i32_i16
                 // multiplies the pair with the channel's weight pair and accumulates (exact, int32).
