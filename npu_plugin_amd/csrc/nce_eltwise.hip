@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
         if (PATH == PATH_HI) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                const uint32_t ua = wa[d] ^ a.in_flip, ub = wb[d] ^ a.in_flip;
+                const uint32_t ua = SIGNED ? wa[d] ^ 0x80808080u : wa[d], ub = SIGNED ? wb[d] ^ 0x80808080u : wb[d];
                 uint32_t packed = 0;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -133,7 +133,7 @@ void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
     if (path == PPE_MODE_FOLDED) launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
     else if (path == PPE_MODE_SLOPE) launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
     else if (path == PPE_MODE_INT) launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
-    else if (path == PATH_HI) hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH_HI, false>), dim3(grid), dim3(256), 0, s, a);
+    else if (path == PATH_HI) launch_signed<FLAT, PATH_HI>(a, grid, s);
     else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
 
