@@ -137,10 +137,16 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
             wsum = ntaps;
         }
     }
-    const bool bad_shift = has_ch && shift > kMaxF64Shift;
-    const bool small_shift = has_ch && ppe_may_saturate((int64_t)ntaps * (MODE == MODE_DW ? 65025 : 255), bias, mult, shift);
-    const bool use_int = __syncthreads_or(bad_shift) != 0;
-    const bool may_sat = __syncthreads_or(small_shift) != 0;
+    // (max pool has no scale: no constants, no workgroup synchronisation)
+    bool use_int = false, may_sat = false;
+    if constexpr (MODE != MODE_MAX) {
+        const bool bad_shift = has_ch && shift > kMaxF64Shift;
+        const bool small_shift = has_ch && ppe_may_saturate((int64_t)ntaps * (MODE == MODE_DW ? 65025 : 255), bias, mult, shift);
+        // (one vote: bit 0 = a shift beyond FP64, bit 1 = possible int32 saturation)
+        const int votes = __syncthreads_or((bad_shift ? 1 : 0) | (small_shift ? 2 : 0));
+        use_int = (votes & 1) != 0;
+        may_sat = (votes & 2) != 0;
+    }
     const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
     const int pmode = ppe_mode_of(pu, use_int);
     if (has_ch) {
@@ -154,7 +160,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         sM[ch] = M;
         sB[ch] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu);
     }
-    __syncthreads();
+    if constexpr (MODE != MODE_MAX) __syncthreads();
 
     const int64_t nitems = a.npix * nslab;
     const int64_t first = (int64_t)xcd_tile(blockIdx.x, a.nblocks) * NT * a.items_per_thread;
