@@ -26,11 +26,11 @@ PEAK_HBM_GBS = 8000.0    # MI355X HBM3E, GB/s
 # Scale factors from the 256 MiB copy in the same runs: FETCH_SIZE reads 131085 KiB for 262144 KiB
 # fetched (x2.0), WRITE_SIZE reads 262144 KiB (x1.0). Values in bytes per launch.
 MEASURED_TRAFFIC = {
-    "cfg2": int((1066.3 * 2.0 + 1568.0) * 1024),
-    "cfg3_dw": int((9491.6 * 2.0 + 4704.0) * 1024),
-    "cfg3_maxpool": int((2406.9 * 2.0 + 1176.0) * 1024),
-    "cfg3_avgpool": int((648.9 * 2.0 + 294.0) * 1024),
-    "cfg4": int((3154.6 * 2.0 + 3136.0) * 1024),
+    "cfg2": int((1056.8 * 2.0 + 1568.0) * 1024),
+    "cfg3_dw": int((9491.2 * 2.0 + 4704.0) * 1024),
+    "cfg3_maxpool": int((2403.9 * 2.0 + 1176.0) * 1024),
+    "cfg3_avgpool": int((646.9 * 2.0 + 294.0) * 1024),
+    "cfg4": int((3154.1 * 2.0 + 3136.0) * 1024),
 }
 
 
