@@ -390,7 +390,9 @@ hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
     if (a.npix == 0 || cgroups == 0) return hipSuccess;
     const int nslabs = (cgroups + SLAB_GROUPS - 1) / SLAB_GROUPS;
     const int64_t items = a.npix * (cgroups < SLAB_GROUPS ? cgroups : SLAB_GROUPS);
-    a.items_per_thread = items > (int64_t)NT * 8192 ? 4 : 1;
+    // (several items per thread amortise the per-workgroup constants of large tasks; max pool has none and measured
+    // fastest with one item per thread at every size)
+    a.items_per_thread = (MODE != MODE_MAX && items > (int64_t)NT * 8192) ? 4 : 1;
     const int64_t blocks = (items + NT * a.items_per_thread - 1) / (NT * a.items_per_thread);
     if (blocks > 0x7ffffff0LL) return hipErrorInvalidValue;
     a.nblocks = (uint32_t)blocks;
