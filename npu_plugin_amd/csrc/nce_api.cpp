@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -15,7 +16,10 @@
 struct nce_executor_s {
     int device = 0;
     nce_log_s* log = nullptr;
+    nce::Options opt;  // tuning knobs, read from the environment once at creation
 };
+
+thread_local nce::LaunchContext nce::tls_launch;
 
 namespace {
 
@@ -32,6 +36,30 @@ struct Plan {
     std::vector<Box> boxes;
     int task_type = 0;
 };
+
+// Sets the calling thread's launch context for the duration of one C-ABI call.
+struct ScopedLaunch {
+    nce::LaunchContext saved;
+    ScopedLaunch(const nce::Options* opt, std::vector<nce::RecordedLaunch>* record) : saved(nce::tls_launch) {
+        nce::tls_launch.opt = opt;
+        nce::tls_launch.record = record;
+    }
+    ~ScopedLaunch() { nce::tls_launch = saved; }
+};
+
+nce::Options read_options() {
+    nce::Options o;
+    if (const char* e = getenv("NCE_HIP_CONV_PATH")) {
+        o.conv_path = atoi(e);
+        o.env_path = true;
+    }
+    if (const char* e = getenv("NCE_HIP_CONV_WRES"))
+        o.wres_forced = sscanf(e, "%d,%d,%d,%d", &o.wres[0], &o.wres[1], &o.wres[2], &o.wres[3]) == 4;
+    if (const char* e = getenv("NCE_HIP_CONV_TILE")) o.halo_tile = atoi(e);
+    if (const char* e = getenv("NCE_HIP_CONV_TILED")) o.tiled = atoi(e);
+    o.no_fuse = getenv("NCE_HIP_NO_FUSE") != nullptr;
+    return o;
+}
 
 #define FAIL(code, ...)              \
     do {                             \
@@ -399,10 +427,45 @@ nce_result_t launch_plan(nce_executor_s* ex, const Plan& plan, hipStream_t strea
 
 }  // namespace
 
+// A task list keeps the validated plans and, from its first Enqueue on, the prepared launches (kernel, grid and
+// argument block of every launch, conv + add pairs already fused): an Enqueue is then a loop of hipLaunchKernel.
 struct nce_task_list_s {
     nce_executor_s* ex = nullptr;
+    std::mutex mu;
     std::vector<Plan> plans;
+    std::vector<nce::RecordedLaunch> launches;
+    bool prepared = false;
 };
+
+namespace {
+
+// Walk the plans the way they are to run (stream order), launching or - with a recorder set - recording.
+nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipStream_t stream) {
+    for (size_t i = 0; i < plans.size(); ++i) {
+        const Plan& p = plans[i];
+        // A convolution directly followed by the residual add that consumes its output runs as one launch where the
+        // kernels allow it (both outputs are written; the bytes are those of the two tasks run one after the other).
+        if (p.task_type == NCE_TASK_CONV && p.boxes.size() == 1 && i + 1 < plans.size()) {
+            const Plan& q = plans[i + 1];
+            if (q.task_type == NCE_TASK_ELTWISE && q.boxes.size() == 1) {
+                const hipError_t e = nce::launch_conv_fused_add(p.dev, p.boxes[0], q.dev, q.boxes[0], stream);
+                if (e == hipSuccess) {
+                    ++i;
+                    continue;
+                }
+                if (e != hipErrorNotSupported) {
+                    ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
+                    return NCE_RESULT_ERROR_UNKNOWN;
+                }
+            }
+        }
+        const nce_result_t r = launch_plan(ex, p, stream);
+        if (r != NCE_RESULT_SUCCESS) return r;
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -427,6 +490,7 @@ nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* 
     lg->level = desc.log_level;
     ex->log = lg;
     ex->device = desc.device_id;
+    ex->opt = read_options();
     if (desc.device_id >= 0) {
         int count = 0;
         const hipError_t e = hipGetDeviceCount(&count);
@@ -474,6 +538,7 @@ nce_result_t nceClusterTaskEnqueue(nce_executor_handle_t executor, const nce_clu
             return NCE_RESULT_ERROR_UNSUPPORTED;
         }
         if (hipSetDevice(executor->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
+        const ScopedLaunch ctx(&executor->opt, nullptr);
         return launch_plan(executor, plan, static_cast<hipStream_t>(hip_stream));
     } catch (const std::bad_alloc&) {
         return NCE_RESULT_ERROR_OUT_OF_MEMORY;
@@ -497,7 +562,10 @@ nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_ta
         Plan plan;
         const nce_result_t r = make_plan(list->ex->log, task, &plan);
         if (r != NCE_RESULT_SUCCESS) return r;
+        std::lock_guard<std::mutex> lk(list->mu);
         list->plans.push_back(std::move(plan));
+        list->prepared = false;
+        list->launches.clear();
         return NCE_RESULT_SUCCESS;
     } catch (const std::bad_alloc&) {
         return NCE_RESULT_ERROR_OUT_OF_MEMORY;
@@ -511,28 +579,32 @@ nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
     if (list->ex->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
     if (hipSetDevice(list->ex->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    for (size_t i = 0; i < list->plans.size(); ++i) {
-        const Plan& p = list->plans[i];
-        // A convolution directly followed by the residual add that consumes its output runs as one launch where the
-        // kernels allow it (both outputs are written; the bytes are those of the two tasks run one after the other).
-        if (p.task_type == NCE_TASK_CONV && p.boxes.size() == 1 && i + 1 < list->plans.size()) {
-            const Plan& q = list->plans[i + 1];
-            if (q.task_type == NCE_TASK_ELTWISE && q.boxes.size() == 1) {
-                const hipError_t e = nce::launch_conv_fused_add(p.dev, p.boxes[0], q.dev, q.boxes[0], stream);
-                if (e == hipSuccess) {
-                    ++i;
-                    continue;
-                }
-                if (e != hipErrorNotSupported) {
-                    list->ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
-                    return NCE_RESULT_ERROR_UNKNOWN;
-                }
+    try {
+        std::lock_guard<std::mutex> lk(list->mu);
+        if (!list->prepared) {
+            // Kernel choice, grids and argument blocks are worked out once, here; later calls only replay them.
+            list->launches.clear();
+            const ScopedLaunch ctx(&list->ex->opt, &list->launches);
+            const nce_result_t r = run_plans(list->ex, list->plans, nullptr);
+            if (r != NCE_RESULT_SUCCESS) {
+                list->launches.clear();
+                return r;
+            }
+            list->prepared = true;
+        }
+        for (const nce::RecordedLaunch& l : list->launches) {
+            const hipError_t e = nce::replay(l, stream);
+            if (e != hipSuccess) {
+                list->ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
+                return NCE_RESULT_ERROR_UNKNOWN;
             }
         }
-        const nce_result_t r = launch_plan(list->ex, p, stream);
-        if (r != NCE_RESULT_SUCCESS) return r;
+        return NCE_RESULT_SUCCESS;
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (...) {
+        return NCE_RESULT_ERROR_UNKNOWN;
     }
-    return NCE_RESULT_SUCCESS;
 }
 
 nce_result_t nceTaskListDestroy(nce_task_list_handle_t list) {

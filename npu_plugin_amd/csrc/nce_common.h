@@ -2,8 +2,10 @@
 #pragma once
 
 #include <atomic>
+#include <cstring>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <vector>
 
 #include "../../include/nce_hip.h"
 
@@ -109,6 +111,61 @@ struct LdsGrant {
         return hipSuccess;
     }
 };
+
+// Tuning / test knobs of an executor. Read from the environment ONCE, when the executor is created
+// (nceExecutorCreate); a launch never calls getenv.
+struct Options {
+    int conv_path = 0;        // NCE_HIP_CONV_PATH: 1 = skip the weights-resident kernel, 2 = gather kernel only
+    bool wres_forced = false; // NCE_HIP_CONV_WRES="nf,bf,nwaves,tiles_per_wave" was given ...
+    int wres[4] = {0, 0, 0, 0};  // ... with these values
+    int halo_tile = -1;       // NCE_HIP_CONV_TILE: force one halo tile shape (0..3)
+    bool no_fuse = false;     // NCE_HIP_NO_FUSE: task lists never run a convolution and the add after it as one launch
+    int tiled = -1;           // NCE_HIP_CONV_TILED: -1 automatic, 0 never, 1.. force that shape of the LDS-tiled kernel
+    bool env_path = false;    // NCE_HIP_CONV_PATH was given at all (switches the conv + add fusion off, as NO_FUSE does)
+};
+
+// One prepared kernel launch: the kernel, its grid and a copy of its (single, by-value) argument struct.
+struct RecordedLaunch {
+    const void* func = nullptr;
+    dim3 grid, block;
+    uint32_t lds = 0;
+    std::vector<uint64_t> arg;  // argument bytes (8-byte aligned storage; the largest member of every argument struct is 8 bytes)
+};
+
+// What a launch_* function needs besides its task: the executor's options and, when a task list prepares its
+// launches, the list to record into instead of launching. Set by the C-ABI entry points around their calls
+// (thread-local: one executor may be used from several host threads).
+struct LaunchContext {
+    const Options* opt = nullptr;
+    std::vector<RecordedLaunch>* record = nullptr;
+};
+extern thread_local LaunchContext tls_launch;
+inline const Options& options() {
+    static const Options defaults;
+    return tls_launch.opt ? *tls_launch.opt : defaults;
+}
+
+// Launch `kernel(arg)` now, or record the launch when a task list is being prepared.
+template <typename Arg>
+inline hipError_t emit(void (*kernel)(Arg), dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Arg& arg) {
+    if (std::vector<RecordedLaunch>* rec = tls_launch.record) {
+        RecordedLaunch r;
+        r.func = reinterpret_cast<const void*>(kernel);
+        r.grid = grid;
+        r.block = block;
+        r.lds = (uint32_t)lds;
+        r.arg.resize((sizeof(Arg) + 7) / 8);
+        memcpy(r.arg.data(), &arg, sizeof(Arg));
+        rec->push_back(std::move(r));
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, arg);
+    return hipGetLastError();
+}
+inline hipError_t replay(const RecordedLaunch& r, hipStream_t stream) {
+    void* args[1] = {const_cast<uint64_t*>(r.arg.data())};
+    return hipLaunchKernel(r.func, r.grid, r.block, args, r.lds, stream);
+}
 
 hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream);
 hipError_t launch_pool(const TaskDev& t, const Box& box, bool is_max, hipStream_t stream);

@@ -226,12 +226,11 @@ hipError_t launch_conv_gather(const ConvArgs& a, hipStream_t stream) {
     if (wg256 >= 512) {
         const int64_t gx = ((int64_t)a.M + 255) / 256;
         if (gx > 0x7fffffffLL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((conv_igemm_kernel<2>), dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
+        return emit(conv_igemm_kernel<2>, dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
     } else {
         const int64_t gx = ((int64_t)a.M + 127) / 128;
-        hipLaunchKernelGGL((conv_igemm_kernel<1>), dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
+        return emit(conv_igemm_kernel<1>, dim3(xcd_grid((unsigned)gx), gy), dim3(NTHREADS), 0, stream, a);
     }
-    return hipGetLastError();
 }
 
 // Launch arguments of a convolution over one box; hipSuccess, or the error to return.
@@ -282,6 +281,7 @@ static hipError_t make_conv_args(const TaskDev& t, const Box& box, ConvArgs& a) 
     a.dw = off_w - t.w_zp;
     const uint32_t fb = (uint32_t)((t.in.zp - off_a) & 0xFF);
     a.fill = fb * 0x01010101u;
+    a.fill_raw = (uint32_t)(t.in.zp & 0xFF);
     a.pitchpx = t.in.w + t.pl + t.pr;
     a.nslots_max = a.rows_max = a.nchunks = a.halo_bytes = 0;
     a.ppe = t.ppe;
@@ -302,8 +302,16 @@ static bool overlaps(const TensorDev& x, const TensorDev& y) {
     return x.data < ye && y.data < xe;
 }
 
+// Which convolutions take the LDS-tiled kernel: 0 = none of its shapes, else the shape (0 within a forced value: automatic).
+static int tiled_shape_for(const ConvArgs& a) {
+    const int forced = options().tiled;
+    if (forced >= 0) return forced;
+    (void)a;
+    return 0;
+}
+
 hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskDev& add, const Box& ab, hipStream_t stream) {
-    if (getenv("NCE_HIP_NO_FUSE") || getenv("NCE_HIP_CONV_PATH")) return hipErrorNotSupported;
+    if (options().no_fuse || options().env_path) return hipErrorNotSupported;
     const TensorDev& o = conv.out;
     const bool conv_full = cb.x0 == 0 && cb.y0 == 0 && cb.z0 == 0 && cb.bw == o.w && cb.bh == o.h && cb.bc == o.c;
     const bool add_full = ab.x0 == 0 && ab.y0 == 0 && ab.z0 == 0 && ab.bw == add.out.w && ab.bh == add.out.h && ab.bc == add.out.c;
@@ -333,6 +341,10 @@ hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskD
     ConvArgs a;
     if (const hipError_t e = make_conv_args(conv, cb, a); e != hipSuccess) return e;
     if (a.M == 0 || cb.bc == 0) return hipErrorNotSupported;
+    if (const int shape = tiled_shape_for(a)) {
+        const hipError_t e = launch_conv_tiled(a, stream, shape, &fz);
+        if (e != hipErrorNotSupported) return e;
+    }
     return launch_conv_wres(a, stream, false, &fz);
 }
 
@@ -341,12 +353,14 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     if (const hipError_t e0 = make_conv_args(t, box, a); e0 != hipSuccess) return e0;
     if (a.M == 0 || box.bc == 0) return hipSuccess;
     // tuning and test knob: 1 = skip the weights-resident kernel, 2 = gather kernel only
-    const char* path_env = getenv("NCE_HIP_CONV_PATH");
-    const int path = path_env ? atoi(path_env) : 0;
+    const int path = options().conv_path;
     // Reductions too long for one LDS slice: the halo kernel is the faster one for 3-wide kernels (measured on
     // 3x3 over 1024 channels), the chunked weights-resident kernel for everything else and for what the halo
     // kernel rejects.
-    hipError_t e = path == 0 ? launch_conv_wres(a, stream, a.KX != 3) : hipErrorNotSupported;
+    hipError_t e = hipErrorNotSupported;
+    if (const int shape = path == 0 ? tiled_shape_for(a) : 0) e = launch_conv_tiled(a, stream, shape);
+    if (e != hipErrorNotSupported) return e;
+    e = path == 0 ? launch_conv_wres(a, stream, a.KX != 3) : hipErrorNotSupported;
     if (e != hipErrorNotSupported) return e;
     e = path <= 1 ? launch_conv_halo(a, stream) : hipErrorNotSupported;
     if (e != hipErrorNotSupported) return e;

@@ -50,6 +50,7 @@ struct ConvArgs {
     int32_t ICG;  // 16-byte groups per tap: IC/16
     uint32_t a_xor, w_xor;  // 0x80808080 for u8 storage, 0 for i8
     uint32_t fill;          // out-of-image activation word, re-biased
+    uint32_t fill_raw;      // the same byte as stored (the input zero point), 0..255
     int32_t da, dw;         // (storage offset - zero point) of activations / weights
     int32_t ktot;           // KY*KX*IC
     // halo kernel only
@@ -213,5 +214,7 @@ struct FuseAdd {
 
 // fuse: optional; hipErrorNotSupported when the kernel variant that would run the task cannot carry the add.
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse = nullptr);
+// LDS-tiled kernel for many output channels; shape 1.. selects a tile shape (see nce_conv_tiled.hip), 0 the automatic choice.
+hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, const FuseAdd* fuse = nullptr);
 
 }  // namespace nce

@@ -55,6 +55,7 @@ __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
     if (tile >= ntiles) return;  // uniform for the whole workgroup
 
     epi_load_table(a, es, tid, NT, BN, oc0, noc);
+    __syncthreads();  // the zeroed weight sums are in place before any wave adds to them (store_weights below)
 
     // ---- tile geometry (uniform) ------------------------------------------------------------
     const int32_t m0 = tile * BM;
@@ -302,8 +303,7 @@ hipError_t try_launch(ConvArgs a, hipStream_t stream, bool* fits) {
     auto kernel = &conv_halo_kernel<WN, WP, AF, BF, KX>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3(xcd_grid((unsigned)gx), gy), dim3(NT), lds, stream, a);
-    return hipGetLastError();
+    return emit(kernel, dim3(xcd_grid((unsigned)gx), gy), dim3(NT), lds, stream, a);
 }
 
 // Tile shapes: {channel waves, pixel waves, channel fragments, pixel fragments per wave}.
@@ -330,10 +330,7 @@ hipError_t launch_kx(const ConvArgs& a, hipStream_t stream) {
     if (KX == 1 && px256 * ch64 >= 384) first = 1;
     (void)px128;
     (void)ch128;
-    static const int forced = [] {
-        const char* e = getenv("NCE_HIP_CONV_TILE");  // tuning knob: force one tile shape (0..3)
-        return e ? atoi(e) : -1;
-    }();
+    const int forced = options().halo_tile;  // tuning knob: force one tile shape (0..3)
     if (forced >= 0 && forced <= 3) first = forced;
     for (int tile = first; tile <= 3; ++tile) {
         bool fits = false;

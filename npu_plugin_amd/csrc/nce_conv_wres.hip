@@ -21,7 +21,7 @@
 // the OYXI weight row, i.e. tap u / (IC/16), input channels 16 * (u % (IC/16)). With IC a multiple of
 // 64 a step never straddles taps and the tap bookkeeping is scalar; other channel counts take the
 // per-lane path (template MODE 2). Semantics and the fused PPE are the ones of nce_conv.hip.
-#include "nce_conv_common.h"
+#include "nce_conv_epi.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -61,6 +61,8 @@ hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, h
 
 namespace {
 
+using namespace wres_detail;
+
 enum { WRES_FAST = 0, WRES_FAST_MASK = 1, WRES_GENERIC = 2 };
 
 // Per reduction step (modes 0 and 1): input byte offset of the step's tap and channel chunk relative to the
@@ -71,169 +73,6 @@ struct __attribute__((aligned(16))) StepEntry {
     int32_t pad;
 };
 constexpr int kMaxSteps = 80;  // 144 KiB / (2 fragments * 1 KiB) = 72 steps, padded to the load depth
-
-// One 64-byte line per byte value: lanes whose tap lies outside the image load the input zero point from
-// here instead of the activation tensor, so every activation load is unconditional (nothing has to
-// wait for it until the matrix instruction that consumes it).
-struct FillTable {
-    uint8_t b[256][64];
-};
-constexpr FillTable make_fill_table() {
-    FillTable t{};
-    for (int v = 0; v < 256; ++v)
-        for (int i = 0; i < 64; ++i) t.b[v][i] = (uint8_t)v;
-    return t;
-}
-// (not const: a constant-address-space pointer selected against a global one would turn every activation load
-// into a FLAT load, which also counts against the LDS wait counter)
-__device__ FillTable g_fill = make_fill_table();
-
-// Channel (within the slice) that row i of channel fragment f carries: lane (c, q) of the result then
-// holds channels 4*NF*q .. 4*NF*q + 4*NF-1, consecutive, for f = 0..NF-1 and its 4 registers.
-template <int NF>
-__device__ __forceinline__ int channel_of_frag_row(int f, int i) {
-    return 4 * NF * (i >> 2) + 4 * f + (i & 3);
-}
-
-// bits [lo, hi) of a 32-bit mask (empty when hi <= lo; hi - lo <= 32)
-__device__ __forceinline__ uint32_t bit_range(int lo, int hi) {
-    return hi > lo ? ((0xFFFFFFFFu >> (32 - (hi - lo))) << lo) : 0u;
-}
-
-// Wave-uniform constants of the FP64 epilogues. Outputs are computed as bytes 0..255: signed outputs 128
-// higher, flipped back by an XOR on the packed word; truncating conversion to int32, one v_med3_i32, byte
-// insert.
-struct EpiPack {
-    int32_t ilo, ihi;   // clamp bounds with the zero point (+128 for signed outputs) added: 0 <= ilo <= ihi <= 255
-    uint32_t flip;      // 0x80808080 for signed outputs
-    double zp_fold;     // what B carries on top of the bias term: the output zero point (+128 for signed outputs)
-    double pcz;         // slope mode: rounding constant of the slope + zp_fold * (1 - slope)
-    int32_t pmq;        // high-word slope mode: slope * 2^32 ...
-    int64_t cpz;        // ... and (rounding constant + zp_fold * (1 - slope)) * 2^32
-};
-
-__device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
-    EpiPack e;
-    const int32_t sb = pu.lo_zp < 0 ? 128 : 0;  // only signed storage clamps below zero
-    e.ilo = pu.lo_zp + sb;
-    e.ihi = pu.hi_zp + sb;
-    e.flip = sb ? 0x80808080u : 0u;
-    e.zp_fold = (double)(pu.zp + sb);
-    e.pcz = pu.pc + e.zp_fold - e.zp_fold * pu.pm;  // exact: 8 integer bits, at most 31 fractional bits
-    e.pmq = 0;
-    e.cpz = 0;
-    return e;
-}
-
-typedef unsigned short fz_u16x2 __attribute__((ext_vector_type(2)));
-
-template <int NF, int BF, int PMODE, bool FZ = false>
-__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
-                                              const v4i (&acc)[NF][BF], const int32_t (&dws)[BF], int q, int noc,
-                                              uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
-                                              const EpiPack& ep, const FuseAdd* fz = nullptr, const uint4* other = nullptr) {
-    const int ch0 = 4 * NF * q;
-    if (ch0 >= noc) return;
-    static_assert(!FZ || NF == 4, "fused add: a lane holds 16 channels");
-    uint32_t wo[BF][NF];
-#pragma unroll
-    for (int f = 0; f < NF; ++f) {
-#pragma unroll
-        for (int x = 0; x < BF; ++x) wo[x][f] = 0;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int c = ch0 + 4 * f + r;
-            double M = 0.0, B = 0.0;
-            int32_t w2 = 0, bias = 0, corr = 0;
-            // (the activation zero point is already in the wave's constants: da * sum of the channel's weights)
-            int32_t mq = 0;
-            int64_t cq = 0;
-            if (PMODE == PPE_MODE_INT) {
-                w2 = s.w2[c];
-                bias = s.bias[c];
-                corr = sCorr[c];
-            } else if (PMODE == PPE_MODE_HI || PMODE == PPE_MODE_HI_SLOPE) {
-                mq = sCorr[c];
-                cq = reinterpret_cast<const int64_t*>(sBfull)[c];
-            } else {
-                M = s.M[c];
-                B = sBfull[c];
-            }
-#pragma unroll
-            for (int x = 0; x < BF; ++x) {
-                const int32_t av = acc[f][x][r] + dws[x];  // (+ dw * sum of the pixel's activations; 0 when dw == 0)
-                if (PMODE == PPE_MODE_INT) {
-                    const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
-                    wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
-                } else if (PMODE == PPE_MODE_HI) {
-                    // y = floor(((av + bias') * mult + 2^(shift-1) + zp * 2^shift) / 2^shift), everything scaled
-                    // by 2^(32 - shift) so that the division is "take the high word": one 32 x 32 + 64 bit
-                    // multiply-add per output. mq and cq are set up per wave (see kernel).
-                    const int32_t y = clamp_med3((int32_t)(((int64_t)av * mq + cq) >> 32), ep.ilo, ep.ihi);
-                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
-                } else if (PMODE == PPE_MODE_HI_SLOPE) {
-                    // The same with a negative slope |slope| <= 1: rz is the value before the slope (zero point
-                    // added), nz the value after it, both exact; the larger of the two is the result (below
-                    // zero the slope raises a value, from zero up it does not).
-                    const int32_t rz = (int32_t)(((int64_t)av * mq + cq) >> 32);
-                    const int32_t nz = (int32_t)(((int64_t)rz * ep.pmq + ep.cpz) >> 32);
-                    const int32_t y = min(max(max(rz, nz), ep.ilo), ep.ihi);
-                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
-                } else if (PMODE == PPE_MODE_FOLDED) {
-                    // The conversion truncates; below zero that differs from floor, but every value below
-                    // zero (and floor's -1 for a value in (-1, 0)) clamps to ep.ilo >= 0 either way.
-                    const int32_t y = clamp_med3((int32_t)__builtin_fma((double)av, M, B), ep.ilo, ep.ihi);
-                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
-                } else {
-                    // Slope mode, everything shifted up by the output zero point zp (B carries it, as in folded
-                    // mode): tz = t + zp. Below zero the slope applies to floor(t) = floor(tz) - zp, which
-                    // ep.pcz folds in: n = floor(t) * pm + pc + zp, exact. Both candidates are converted by
-                    // truncation - right for values >= 0, and below 0 everything clamps to ep.ilo >= 0.
-                    const double tz = __builtin_fma((double)av, M, B);
-                    const double n = __builtin_fma(__builtin_floor(tz), pu.pm, ep.pcz);
-                    const int32_t y = clamp_med3(tz < ep.zp_fold ? (int32_t)n : (int32_t)tz, ep.ilo, ep.ihi);
-                    wo[x][f] = r == 0 ? (uint32_t)y : (wo[x][f] | ((uint32_t)y << (8 * r)));
-                }
-            }
-        }
-        if (PMODE != PPE_MODE_INT) {
-#pragma unroll
-            for (int x = 0; x < BF; ++x) wo[x][f] ^= ep.flip;
-        }
-        __builtin_amdgcn_sched_barrier(0);  // one fragment's constants live at a time
-    }
-#pragma unroll
-    for (int x = 0; x < BF; ++x) {
-        if (!valid[x]) continue;
-        if constexpr (NF == 4) store_channels16(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1], wo[x][2], wo[x][3]);
-        else store_channels8(dst[x] + ch0 * a.out_sc, a.out_sc, wo[x][0], wo[x][1]);
-    }
-    if constexpr (FZ) {
-        // The add on the bytes just stored (a.out_sc == 1 here): byte i of both inputs as a pair of 16-bit values, one
-        // 16-bit dot product with the two input multipliers, the high word of one multiply-add, clamp, byte insert.
-#pragma unroll
-        for (int x = 0; x < BF; ++x) {
-            if (!valid[x]) continue;
-            const uint32_t ob[4] = {other[x].x, other[x].y, other[x].z, other[x].w};
-            uint32_t r[4];
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const uint32_t ua = wo[x][d] ^ fz->in_flip, ub = ob[d] ^ fz->in_flip;
-                uint32_t packed = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t pair = __builtin_amdgcn_perm(ub, ua, 0x0c040c00u + (uint32_t)i * 0x00010001u);
-                    const int32_t sum = (int32_t)__builtin_amdgcn_udot2(__builtin_bit_cast(fz_u16x2, pair), __builtin_bit_cast(fz_u16x2, fz->mults),
-                                                                         (uint32_t)fz->c0h, false);
-                    const int32_t y = clamp_med3((int32_t)(((int64_t)sum * fz->mq + fz->cq) >> 32), fz->ilo, fz->ihi);
-                    packed = i == 0 ? (uint32_t)y : (packed | ((uint32_t)y << (8 * i)));
-                }
-                r[d] = packed ^ fz->flip;
-            }
-            *reinterpret_cast<uint4*>(fz->out + ((dst[x] + ch0) - a.out)) = make_uint4(r[0], r[1], r[2], r[3]);
-        }
-    }
-}
 
 // D: reduction steps whose activation loads are in flight per wave; the host picks a D that divides the step
 // count where it can and pads the step count otherwise (a padding step multiplies zero weights).
@@ -744,8 +583,7 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     auto kernel = &conv_wres_kernel<NF, BF, MODE, D, LM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
-    return hipGetLastError();
+    return emit(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
 }
 
 template <int NF, int BF, int D>
@@ -1119,8 +957,7 @@ hipError_t launch_chunked(WresArgs& w, int nwaves, hipStream_t stream) {
     auto kernel = &conv_wres_chunked_kernel<NF, BF, ASUM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
-    return hipGetLastError();
+    return emit(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
 }
 
 // Long reductions: 32 channels x 72 steps per chunk; the pixel tile as large as still gives ~1500 wave tiles.
@@ -1132,12 +969,10 @@ hipError_t launch_conv_wres_chunked(WresArgs& w, hipStream_t stream) {
     const int64_t slices = (a.bc + 31) / 32;
     int bf = (((int64_t)a.M + 31) / 32) * slices >= 1500 ? 2 : 1;
     int nw = 8;
-    if (const char* forced = getenv("NCE_HIP_CONV_WRES")) {  // "nf,bf,nwaves,tiles_per_wave": bf (1, 2) and nwaves apply
-        int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
-        if (sscanf(forced, "%d,%d,%d,%d", &fnf, &fbf, &fnw, &ftpw) == 4) {
-            if (fbf == 1 || fbf == 2) bf = fbf;
-            if (fnw >= 1 && fnw <= 8) nw = fnw;
-        }
+    if (options().wres_forced) {  // "nf,bf,nwaves,tiles_per_wave": bf (1, 2) and nwaves apply
+        const int fbf = options().wres[1], fnw = options().wres[2];
+        if (fbf == 1 || fbf == 2) bf = fbf;
+        if (fnw >= 1 && fnw <= 8) nw = fnw;
     }
     if (a.dw != 0) return bf == 2 ? launch_chunked<2, 2, true>(w, nw, stream) : launch_chunked<2, 1, true>(w, nw, stream);
     return bf == 2 ? launch_chunked<2, 2, false>(w, nw, stream) : launch_chunked<2, 1, false>(w, nw, stream);
@@ -1231,15 +1066,12 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
 
     int nw = nwaves;
     bool forced_tpw = false;
-    const char* forced = getenv("NCE_HIP_CONV_WRES");  // tuning and test knob: "nf,bf,nwaves,tiles_per_wave"
-    if (forced) {
-        int fnf = 0, fbf = 0, fnw = 0, ftpw = 0;
-        if (sscanf(forced, "%d,%d,%d,%d", &fnf, &fbf, &fnw, &ftpw) == 4) {
-            if ((fnf == 2 || (fnf == 4 && wl4 <= kWresLdsCap))) nf = fnf;
-            if (fbf == 1 || fbf == 2 || fbf == 4) bf = fbf;
-            if (fnw >= 1 && fnw <= 8) nw = fnw;
-            if (ftpw >= 1) tpw = ftpw, forced_tpw = true;  // (0: keep the automatic choice below)
-        }
+    if (options().wres_forced) {  // tuning and test knob: "nf,bf,nwaves,tiles_per_wave"
+        const int fnf = options().wres[0], fbf = options().wres[1], fnw = options().wres[2], ftpw = options().wres[3];
+        if ((fnf == 2 || (fnf == 4 && wl4 <= kWresLdsCap))) nf = fnf;
+        if (fbf == 1 || fbf == 2 || fbf == 4) bf = fbf;
+        if (fnw >= 1 && fnw <= 8) nw = fnw;
+        if (ftpw >= 1) tpw = ftpw, forced_tpw = true;  // (0: keep the automatic choice below)
     }
     if (w.fused && nf4_ok) nf = 4;  // (the fused add exists for the 64-channel kernels)
     w.tpg = forced_tpw ? 0 : pick_tpg(nf, bf, nw);

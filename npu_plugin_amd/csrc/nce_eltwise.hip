@@ -123,18 +123,18 @@ bool is_dense_nhwc(const TensorDev& x) {
 }
 
 template <bool FLAT, int PATH>
-void launch_signed(const EltArgs& a, int grid, hipStream_t s) {
-    if (a.t.in.is_signed) hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH, true>), dim3(grid), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((eltwise_kernel<FLAT, PATH, false>), dim3(grid), dim3(256), 0, s, a);
+hipError_t launch_signed(const EltArgs& a, int grid, hipStream_t s) {
+    if (a.t.in.is_signed) return emit(eltwise_kernel<FLAT, PATH, true>, dim3(grid), dim3(256), 0, s, a);
+    return emit(eltwise_kernel<FLAT, PATH, false>, dim3(grid), dim3(256), 0, s, a);
 }
 
 template <bool FLAT>
-void launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
-    if (path == PPE_MODE_FOLDED) launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
-    else if (path == PPE_MODE_SLOPE) launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
-    else if (path == PPE_MODE_INT) launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
-    else if (path == PATH_HI) launch_signed<FLAT, PATH_HI>(a, grid, s);
-    else launch_signed<FLAT, PATH_TABLE>(a, grid, s);
+hipError_t launch_path(const EltArgs& a, int path, int grid, hipStream_t s) {
+    if (path == PPE_MODE_FOLDED) return launch_signed<FLAT, PPE_MODE_FOLDED>(a, grid, s);
+    if (path == PPE_MODE_SLOPE) return launch_signed<FLAT, PPE_MODE_SLOPE>(a, grid, s);
+    if (path == PPE_MODE_INT) return launch_signed<FLAT, PPE_MODE_INT>(a, grid, s);
+    if (path == PATH_HI) return launch_signed<FLAT, PATH_HI>(a, grid, s);
+    return launch_signed<FLAT, PATH_TABLE>(a, grid, s);
 }
 
 
@@ -209,9 +209,7 @@ hipError_t launch_eltwise(const TaskDev& t, const Box& box, hipStream_t stream) 
     const int path = prepare(t, a);
     int64_t blocks = (a.nchunks + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    if (flat) launch_path<true>(a, path, (int)blocks, stream);
-    else launch_path<false>(a, path, (int)blocks, stream);
-    return hipGetLastError();
+    return flat ? launch_path<true>(a, path, (int)blocks, stream) : launch_path<false>(a, path, (int)blocks, stream);
 }
 
 }  // namespace nce

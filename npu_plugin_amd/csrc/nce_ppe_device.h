@@ -12,14 +12,16 @@
 //                      M = mult * 2^-shift and B = bias * M + 1/2, the quantity acc * M + B equals
 //                      N / 2^shift for an integer |N| < 2^53 whenever shift <= 52, so one FMA
 //                      returns it without rounding and floor() (or rint() for ties-to-even) is the
-//                      integer pipeline's rounding shift. Shifts above 52 take the integer path.
+//                      integer pipeline's rounding shift. The kernels also fold the output zero point
+//                      (up to 8 more integer bits: zp * 2^shift joins N) into B, so the limit they use
+//                      is shift <= 44; larger shifts take the integer path.
 #pragma once
 
 #include "nce_common.h"
 
 namespace nce {
 
-constexpr int kMaxF64Shift = 52;  // largest shift for which the FP64 formulation is exact
+constexpr int kMaxF64Shift = 44;  // largest shift for which the FP64 formulation, zero point folded in, is exact
 
 // Can round_shift((acc + bias) * mult, shift) leave int32 for any |acc| <= acc_bound ?
 // (It cannot once shift >= 18, because |x * mult| < 2^48; smaller shifts are fine for small sums.)

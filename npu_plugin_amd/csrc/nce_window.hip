@@ -376,8 +376,7 @@ template <int MODE, int KK, bool I32>
 hipError_t launch_window_i32(const WinArgs& a, int64_t blocks, int nslabs, size_t lds, hipStream_t s) {
     static LdsGrant grant;  // large depthwise kernels: opt in to more than the default dynamic LDS
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(&window_kernel<MODE, KK, I32>), lds, 32 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL((window_kernel<MODE, KK, I32>), dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
-    return hipGetLastError();
+    return emit(window_kernel<MODE, KK, I32>, dim3(xcd_grid((unsigned)blocks), (unsigned)nslabs), dim3(NT), lds, s, a);
 }
 
 template <int MODE, int KK>

@@ -28,3 +28,24 @@ def validator():
     ex = nce.Executor(device_id=-1, log_level=2)
     yield ex
     ex.destroy()
+
+
+@pytest.fixture
+def tuned(monkeypatch):
+    """Factory of executors created with tuning knobs in the environment (the library reads them once, when an
+    executor is created): tuned(NCE_HIP_CONV_WRES="4,2,8,1") -> executor."""
+    import npu_plugin_amd as nce
+    made = []
+
+    def make(**env):
+        for k, v in env.items():
+            monkeypatch.setenv(k, str(v))
+        ex = nce.Executor(device_id=0, log_level=2)
+        for k in env:
+            monkeypatch.delenv(k)
+        made.append(ex)
+        return ex
+
+    yield make
+    for ex in made:
+        ex.destroy()

@@ -234,7 +234,7 @@ def test_task_list_chain(executor):
 
 # ---- cfg5: the ResNet-50 task graph ---------------------------------------------------------------
 
-@pytest.mark.parametrize("batch,size", [(1, 224), (3, 96)])
+@pytest.mark.parametrize("batch,size", [(3, 96)])
 def test_resnet50_graph_every_tensor(executor, batch, size):
     """All 70 tasks (53 convs, max pool, 16 adds) chained on the GPU through one task list; every
     intermediate tensor must equal the oracle's, not just the last one."""
@@ -275,16 +275,16 @@ WRES_SHAPES = [
 
 @pytest.mark.parametrize("config", WRES_CONFIGS)
 @pytest.mark.parametrize("shape", WRES_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
-def test_conv_weights_resident_instantiations(executor, monkeypatch, shape, config):
+def test_conv_weights_resident_instantiations(tuned, shape, config):
     n, h, w, ic, oc, k, s, pads, in_zp = shape
-    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    executor = tuned(NCE_HIP_CONV_WRES=config)
     check(K.conv_case(400 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=in_zp, out_zp=9,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
 
 
 @pytest.mark.parametrize("config", ["4,2,8,1", "2,1,4,2"])
-def test_conv_weights_resident_types_and_modes(executor, monkeypatch, config):
-    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+def test_conv_weights_resident_types_and_modes(tuned, config):
+    executor = tuned(NCE_HIP_CONV_WRES=config)
     check(K.conv_case(421, 2, 14, 14, 64, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128), executor)
     check(K.conv_case(422, 2, 14, 14, 64, 64, w_signed=False, w_zp=128, in_zp=121), executor)
     check(K.conv_case(423, 2, 14, 14, 64, 64, in_zp=3, ppe=dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255,
@@ -315,17 +315,17 @@ WZP_SHAPES = [
 
 @pytest.mark.parametrize("config", ["4,4,8,1", "4,2,8,2", "4,1,4,1", "2,2,4,3", "2,1,8,1"])
 @pytest.mark.parametrize("shape", WZP_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
-def test_conv_weights_resident_weight_zero_point(executor, monkeypatch, shape, config):
+def test_conv_weights_resident_weight_zero_point(tuned, shape, config):
     n, h, w, ic, oc, k, s, pads = shape
-    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    executor = tuned(NCE_HIP_CONV_WRES=config)
     # u8 weights around 117 (offset +11 from the re-biased storage), then i8 weights with zero point 5
     check(K.conv_case(600 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=131, w_signed=False, w_zp=117, out_zp=9,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
     check(K.conv_case(700 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_signed=True, in_zp=-3, w_signed=True, w_zp=5), executor)
 
 
-def test_conv_weights_resident_variants(executor, monkeypatch):
-    monkeypatch.setenv("NCE_HIP_CONV_WRES", "2,2,4,1")
+def test_conv_weights_resident_variants(tuned):
+    executor = tuned(NCE_HIP_CONV_WRES="2,2,4,1")
     test_conv_halo_variants(executor)
     test_conv_halo_variants(executor, ic=128)   # permuted activation loads, boxes that start inside the image
 
@@ -334,13 +334,13 @@ def test_conv_weights_resident_variants(executor, monkeypatch):
 # (the dispatcher prefers the weights-resident kernel; NCE_HIP_CONV_PATH=1 sends these to the halo kernel)
 
 @pytest.fixture
-def halo_path(monkeypatch):
-    monkeypatch.setenv("NCE_HIP_CONV_PATH", "1")
+def halo_path(tuned):
+    return tuned(NCE_HIP_CONV_PATH="1")
 
 
 @pytest.fixture
-def gather_path(monkeypatch):
-    monkeypatch.setenv("NCE_HIP_CONV_PATH", "2")
+def gather_path(tuned):
+    return tuned(NCE_HIP_CONV_PATH="2")
 
 
 HALO_CASES = [
@@ -364,13 +364,15 @@ HALO_CASES = [
 
 
 @pytest.mark.parametrize("shape", HALO_CASES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}s{s[6][0]}")
-def test_conv_halo_kernel_shapes(executor, halo_path, shape):
+def test_conv_halo_kernel_shapes(halo_path, shape):
+    executor = halo_path
     n, h, w, ic, oc, k, s, pads = shape
     check(K.conv_case(200 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14)), executor)
 
 
-def test_conv_halo_zero_points_and_types(executor, halo_path):
+def test_conv_halo_zero_points_and_types(halo_path):
+    executor = halo_path
     check(K.conv_case(301, 2, 20, 20, 64, 64, in_zp=3, out_zp=17), executor)                      # weight-sum correction
     check(K.conv_case(302, 2, 20, 20, 128, 64, in_signed=True, in_zp=-7, out_signed=True, out_zp=-128), executor)
     check(K.conv_case(303, 2, 20, 20, 64, 64, w_signed=False, w_zp=128, in_zp=121), executor)
@@ -390,13 +392,14 @@ def test_conv_halo_variants(executor, ic=64):
     assert np.array_equal(K.run_hip(part, executor), canvas)
 
 
-def test_conv_halo_variants_on_halo_path(executor, halo_path):
-    test_conv_halo_variants(executor)
+def test_conv_halo_variants_on_halo_path(halo_path):
+    test_conv_halo_variants(halo_path)
 
 
 @pytest.mark.parametrize("shape", [HALO_CASES[3], HALO_CASES[6], HALO_CASES[10], HALO_CASES[12]],
                          ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}s{s[6][0]}")
-def test_conv_gather_kernel_shapes(executor, gather_path, shape):
+def test_conv_gather_kernel_shapes(gather_path, shape):
+    executor = gather_path
     n, h, w, ic, oc, k, s, pads = shape
     check(K.conv_case(500 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=77,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, lrelu_mult=1638, lrelu_shift=14)), executor)
@@ -441,7 +444,7 @@ def test_odu_permutation_conv(executor, order):
 
 
 @pytest.mark.parametrize("order", ["nchw", "nwch", "nhcw"])
-def test_odu_permutation_other_tasks(executor, order, monkeypatch):
+def test_odu_permutation_other_tasks(executor, order, tuned):
     cases = [K.conv_case(601, 1, 9, 9, 16, 32, k=(5, 5), pads=(2, 2, 2, 2)),            # per-lane tap path
              K.dw_case(602, 2, 13, 13, 32), K.pool_case(603, True, 2, 12, 12, 32), K.pool_case(604, False, 2, 12, 12, 32),
              K.eltwise_case(605, 2, 9, 7, 48)]
@@ -449,8 +452,7 @@ def test_odu_permutation_other_tasks(executor, order, monkeypatch):
         got, want = _permuted_run(case, order, executor)
         assert np.array_equal(got, want), case.name
     for path in ("1", "2"):  # halo and gather kernels
-        monkeypatch.setenv("NCE_HIP_CONV_PATH", path)
-        got, want = _permuted_run(K.conv_case(606, 2, 10, 10, 64, 64), order, executor)
+        got, want = _permuted_run(K.conv_case(606, 2, 10, 10, 64, 64), order, tuned(NCE_HIP_CONV_PATH=path))
         assert np.array_equal(got, want), f"conv path {path}"
 
 
@@ -474,9 +476,9 @@ LONG_K_SHAPES = [
 
 @pytest.mark.parametrize("config", ["2,1,8,1", "2,2,4,1", "2,1,3,1"])
 @pytest.mark.parametrize("shape", LONG_K_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
-def test_conv_long_reduction(executor, monkeypatch, shape, config):
+def test_conv_long_reduction(tuned, shape, config):
     n, h, w, ic, oc, k, s, pads = shape
-    monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+    executor = tuned(NCE_HIP_CONV_WRES=config)
     check(K.conv_case(800 + ic + oc + h, n, h, w, ic, oc, k=k, s=s, pads=pads, in_zp=119, out_zp=3,
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
     # weights whose zero point is not their storage offset
@@ -623,7 +625,7 @@ HI_SLOPES = [dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255),
 
 
 @pytest.mark.parametrize("ppe", HI_SLOPES, ids=lambda p: f"m{p.get('lrelu_mult', '-')}s{p.get('lrelu_shift', '-')}")
-@pytest.mark.parametrize("shift", [1, 15, 16, 17, 24, 31, 32, 33, 40])
+@pytest.mark.parametrize("shift", [1, 15, 16, 17, 24, 31, 32, 33, 40, 44, 45, 46, 52, 53])
 def test_conv_epilogue_shift_boundaries(executor, ppe, shift):
     # Every channel of a slice with the same shift: the integer high-word epilogue serves 16/17..32 (the multiplier
     # must fit 31 bits after scaling), FP64 or the 64-bit integer path the rest. Multipliers and biases at their
@@ -663,14 +665,16 @@ def test_eltwise_integer_path_boundaries(executor, signed, shift, mult):
                              mult=mult, shift=shift), executor)
 
 
-def _conv_then_add(executor, monkeypatch, conv_kw, add_kw, conv_first, in_place, config="4,2,8,0", fuse=True):
+def _conv_then_add(tuned, conv_kw, add_kw, conv_first, in_place, config="4,2,8,0", fuse=True, **more_env):
     """A convolution directly followed by the add that reads its output, through one task list; returns the two
     outputs from the GPU and from the oracle."""
     import torch
+    env = dict(more_env)
     if config:
-        monkeypatch.setenv("NCE_HIP_CONV_WRES", config)
+        env["NCE_HIP_CONV_WRES"] = config
     if not fuse:
-        monkeypatch.setenv("NCE_HIP_NO_FUSE", "1")
+        env["NCE_HIP_NO_FUSE"] = "1"
+    executor = tuned(**env)
     c1 = K.conv_case(**conv_kw)
     y1 = K.run_oracle(c1)
     n, h, w, c = c1.out_shape
@@ -697,7 +701,7 @@ def _conv_then_add(executor, monkeypatch, conv_kw, add_kw, conv_first, in_place,
 
 @pytest.mark.parametrize("conv_first,in_place", [(True, False), (False, False), (True, True), (False, True)])
 @pytest.mark.parametrize("config", ["4,4,8,0", "4,2,8,0", "4,1,8,0", "2,2,8,0", None])
-def test_conv_with_fused_residual_add(executor, monkeypatch, conv_first, in_place, config):
+def test_conv_with_fused_residual_add(tuned, conv_first, in_place, config):
     # 1x1 convolutions that close a residual block, followed by the block's add: one launch for both on the 64-channel
     # kernels (a 32-channel configuration and the automatic choice fall back to two launches where they must).
     for ic, oc, out_signed, out_zp in ((64, 256, False, 128), (128, 80, True, -3), (256, 64, False, 0), (512, 128, False, 7)):
@@ -706,22 +710,21 @@ def test_conv_with_fused_residual_add(executor, monkeypatch, conv_first, in_plac
                        ppe=dict(mode=nce.PPE_NOOP, clamp_low=lo + 5, clamp_high=hi))
         add_kw = dict(zp_a=out_zp, zp_b=(out_zp + 9) if not out_signed else -20, out_zp=out_zp, in1_mult=20971, in2_mult=31457,
                       mult=25600, shift=30)
-        g1, g2, y1, y2 = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, conv_first, in_place, config)
+        g1, g2, y1, y2 = _conv_then_add(tuned, conv_kw, add_kw, conv_first, in_place, config)
         assert np.array_equal(g1, y1), "convolution output"
         assert np.array_equal(g2, y2), "add output"
 
 
-def test_conv_fused_add_equals_two_launches(executor, monkeypatch):
+def test_conv_fused_add_equals_two_launches(tuned):
     # the same pair with the fusion switched off, and pairs the fusion must refuse (a 3x3 with padding, an add with a slope)
     conv_kw = dict(seed=7200, n=1, h=14, w=14, ic=128, oc=192, k=(1, 1), pads=(0, 0, 0, 0))
     add_kw = dict(zp_a=128, zp_b=100, out_zp=120)
-    a = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, True, False, "4,2,8,0", fuse=True)
-    b = _conv_then_add(executor, monkeypatch, conv_kw, add_kw, True, False, "4,2,8,0", fuse=False)
+    a = _conv_then_add(tuned, conv_kw, add_kw, True, False, "4,2,8,0", fuse=True)
+    b = _conv_then_add(tuned, conv_kw, add_kw, True, False, "4,2,8,0", fuse=False)
     for x, y in zip(a, b):
         assert np.array_equal(x, y)
-    monkeypatch.delenv("NCE_HIP_NO_FUSE")
     for conv_kw2, add_kw2 in ((dict(conv_kw, k=(3, 3), pads=(1, 1, 1, 1)), add_kw),
                               (conv_kw, dict(add_kw, ppe_extra=dict(mode=nce.PPE_LPRELU, lrelu_mult=1638, lrelu_shift=14))),
                               (conv_kw, dict(add_kw, shift=40))):
-        g1, g2, y1, y2 = _conv_then_add(executor, monkeypatch, conv_kw2, add_kw2, False, False, "4,2,8,0")
+        g1, g2, y1, y2 = _conv_then_add(tuned, conv_kw2, add_kw2, False, False, "4,2,8,0")
         assert np.array_equal(g1, y1) and np.array_equal(g2, y2)
