@@ -70,7 +70,8 @@ typedef enum nce_mpe_mode_t {
     NCE_MPE_NOP = 6
 } nce_mpe_mode_t;
 
-typedef enum nce_dtype_t { NCE_DT_U8 = 0, NCE_DT_I8 = 1, NCE_DT_SI32 = 2 } nce_dtype_t;
+/* F16 / BF16 name float outputs for the parameter generators (nce_params.h) only: tasks with such tensors are rejected. */
+typedef enum nce_dtype_t { NCE_DT_U8 = 0, NCE_DT_I8 = 1, NCE_DT_SI32 = 2, NCE_DT_F16 = 3, NCE_DT_BF16 = 4 } nce_dtype_t;
 
 /* Rounding of the fixed-point right shift in the PPE (requantize and PReLU steps).
  * HALF_UP : (p + 2^(s-1)) >> s, ties toward +inf (default).  HALF_EVEN: ties to even.  NONE: floor. */

@@ -84,6 +84,10 @@ nce_result_t nceHwtestGetScales(nce_hwtest_case_handle_t hw_case, int32_t which,
  * `table` receives OC rows of 4 int32 when the builder emits a weights table (CONV, DWCONV; pools / eltwise only
  * for per-channel output scales); *table_rows tells how many rows were written (0 = no table).
  * Depthwise weights are described in their padded memory form [C, 16 * ceil(KY*KX / 16)].
+ * A ZMajorConvolution whose input channels are no multiple of 16 is described over PADDED buffers, as its builder
+ * allocates them (buildZMConvTest.cpp:111-136): desc->input.dims[1] and desc->weights.dims[1] are the channel count
+ * rounded up to 16; the caller supplies weights whose padding channels hold the weights' zero point (any bytes may
+ * sit in the padding channels of the input).
  * Returns NCE_RESULT_ERROR_UNSUPPORTED for case types, data types or activations the executor cannot run (the log
  * names which). */
 nce_result_t nceHwtestBuildTask(nce_hwtest_case_handle_t hw_case, nce_cluster_task_desc_t* desc, nce_dpu_task_t* variant,

@@ -62,6 +62,27 @@ nce_result_t ncePpeForAvgPool(int32_t arch, nce_quant_t in, nce_quant_t out, int
 nce_result_t ncePpeForEltwiseAdd(int32_t arch, nce_quant_t in1, nce_quant_t in2, nce_quant_t out, int32_t postop,
                                  double p0, double p1, nce_ppe_task_t* ppe);
 
+/* FuseClamp: fold a Clamp {min, max} that follows an NCE op into the op's PPE attributes -
+ * ClampConverter::getTargetClamps and getPPEMode,
+ * src/vpux_compiler/src/dialect/VPU/transforms/passes/fuse_clamp.cpp:34-83. ppe is read and rewritten.
+ * out.dtype U8 / I8 (per-tensor quantized): clamp_low = max(clamp_low, round(min / scale) + zp), clamp_high =
+ * min(clamp_high, round(max / scale) + zp), mode unchanged. out.dtype F16 / BF16: clamp_low = INT32_MIN, clamp_high =
+ * min(clamp_high, bits of max in that type), mode LRELUX. Returns ERROR_UNSUPPORTED, ppe untouched, where the reference
+ * keeps the Clamp as an op of its own (isLegalClamp, fuse_clamp.cpp:123-147): a float output with min != 0. */
+nce_result_t ncePpeFuseClamp(nce_quant_t out, double clamp_min, double clamp_max, nce_ppe_task_t* ppe);
+
+/* Bytes of one output channel's weight set and of the zero padding that completes it to a multiple of 16 bytes:
+ * IC*KY*KX elements are flattened to [OC, 1, 1, IC*KY*KX] and padded when that count is no multiple of 16
+ * (alignConvWeightsTensor, src/vpux_compiler/src/dialect/VPU/utils/const_utils.cpp:245-285; the step of the weight
+ * table pointers, getWeightPtrStep, src/vpux_compiler/src/dialect/VPU/utils/nce_sparsity.cpp:388-413). */
+nce_result_t nceConvWeightSetBytes(int64_t ic, int64_t ky, int64_t kx, int64_t* set_bytes, int64_t* pad_bytes);
+
+/* Check words [0] and [1] of a HOST copy of a weight table against the contract the executor relies on: word [0] of
+ * row oc equals word [0] of row 0 plus oc * weights_ptr_step, every pointer a multiple of 16
+ * (nce_sparsity.cpp:504-510), word [1] the dense marker 0xFFFFFF (nce_sparsity.hpp:32). The executor itself never
+ * dereferences device memory on the host, so it cannot make this check; callers that build tables do. */
+nce_result_t nceWeightsTableCheck(const int32_t* table, int32_t oc, int32_t weights_ptr_step);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,7 +35,7 @@ PPE_NOOP, PPE_ADD, PPE_LRELU, PPE_LRELUX, PPE_LPRELU = 3, 5, 13, 14, 15
 # nce_mpe_mode_t = VPU::MPEMode
 MPE_VECTOR, MPE_MATRIX, MPE_VECTOR_FP16, MPE_CUBOID_16x16, MPE_CUBOID_8x16, MPE_CUBOID_4x16, MPE_NOP = range(7)
 # nce_dtype_t
-DT_U8, DT_I8, DT_SI32 = 0, 1, 2
+DT_U8, DT_I8, DT_SI32, DT_F16, DT_BF16 = 0, 1, 2, 3, 4
 # nce_round_mode_t / nce_clamp_domain_t
 ROUND_HALF_UP, ROUND_HALF_EVEN, ROUND_NONE = 0, 1, 2
 CLAMP_POST_ZP, CLAMP_PRE_ZP = 0, 1
@@ -207,6 +207,9 @@ SYMBOLS = {
     "ncePpeForAvgPool": (C.c_int, [C.c_int32, Quant, Quant, C.c_int32, C.c_int32, C.c_int32, C.c_double, C.c_double,
                                    _P(PpeTask)]),
     "ncePpeForEltwiseAdd": (C.c_int, [C.c_int32, Quant, Quant, Quant, C.c_int32, C.c_double, C.c_double, _P(PpeTask)]),
+    "ncePpeFuseClamp": (C.c_int, [Quant, C.c_double, C.c_double, _P(PpeTask)]),
+    "nceConvWeightSetBytes": (C.c_int, [C.c_int64, C.c_int64, C.c_int64, _P(C.c_int64), _P(C.c_int64)]),
+    "nceWeightsTableCheck": (C.c_int, [_P(C.c_int32), C.c_int32, C.c_int32]),
     "nceHwtestParse": (C.c_int, [C.c_char_p, _P(C.c_void_p), C.c_void_p]),
     "nceHwtestDestroy": (C.c_int, [C.c_void_p]),
     "nceHwtestGetCase": (C.c_int, [C.c_void_p, _P(HwtestCase)]),

@@ -115,9 +115,22 @@ nce_result_t check_activation(nce_log_s* log, const char* name, const nce_tensor
             FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
     } else {
         if (x.strides_bytes[1] != 1) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: layout must be NHWC with compact channels (C stride %lld)", name, (long long)x.strides_bytes[1]);
-        if (x.strides_bytes[3] < x.dims[1] || x.strides_bytes[2] < x.strides_bytes[3] * 1 || x.strides_bytes[0] < x.strides_bytes[2])
-            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides are not NHWC-ordered (N %lld, H %lld, W %lld, C 1)", name,
-                 (long long)x.strides_bytes[0], (long long)x.strides_bytes[2], (long long)x.strides_bytes[3]);
+        // ordered and non-overlapping: a pixel holds C bytes, a row W pixels, an image H rows (extent-1 dimensions aside);
+        // the same size cap as for outputs
+        const int64_t sw = x.strides_bytes[3], sh = x.strides_bytes[2], sn = x.strides_bytes[0];
+        const bool ok_w = x.dims[3] == 1 || sw >= x.dims[1];
+        const bool ok_h = x.dims[2] == 1 || (sh >= x.dims[1] && (x.dims[3] == 1 || sh / x.dims[3] >= sw));
+        const bool ok_n = x.dims[0] == 1 || (sn >= x.dims[1] && (x.dims[3] == 1 || sn / x.dims[3] >= sw) && (x.dims[2] == 1 || sn / x.dims[2] >= sh));
+        if (!ok_w || !ok_h || !ok_n)
+            FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: strides are not NHWC-ordered without overlap (N %lld, H %lld, W %lld, C 1)", name,
+                 (long long)sn, (long long)sh, (long long)sw);
+        int64_t span = x.dims[1];
+        const int64_t ext[3] = {x.dims[3], x.dims[2], x.dims[0]}, str[3] = {sw, sh, sn};
+        for (int i = 0; i < 3; ++i) {
+            if (ext[i] > 1 && (str[i] > 0x7fffffff00LL / (ext[i] - 1))) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: tensor too large", name);
+            span += (ext[i] - 1) * str[i];
+        }
+        if (span > 0x7fffffff00LL) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "%s: tensor too large", name);
         if (((uintptr_t)x.data | (uintptr_t)x.strides_bytes[0] | (uintptr_t)x.strides_bytes[2] | (uintptr_t)x.strides_bytes[3]) & 15)
             FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "%s: data pointer and N/H/W strides must be 16-byte aligned", name);
     }

@@ -118,7 +118,18 @@ private:
         }
         return false;
     }
+    // Nesting is bounded: value() recurses per level, and a descriptor of thousands of '[' must end as a parse error,
+    // not as a stack overflow that no catch block can turn into a result code.
+    static constexpr int kMaxDepth = 64;
+    int depth_ = 0;
+    struct DepthGuard {
+        int& d;
+        explicit DepthGuard(int& depth) : d(depth) { ++d; }
+        ~DepthGuard() { --d; }
+    };
     JValue value() {
+        const DepthGuard guard(depth_);
+        if (depth_ > kMaxDepth) fail("nesting deeper than 64 levels");
         ws();
         if (p_ >= s_.size()) fail("unexpected end of text");
         JValue v;
@@ -659,21 +670,28 @@ void build(const nce_hwtest_case_s& c, nce_cluster_task_desc_t* d, nce_dpu_task_
         if (p.group != 1) throw Unsupported("conv_op.group must be 1 for a ZMajorConvolution");
         if (p.dilation != 1) throw Unsupported("conv_op.dilation must be 1");
         if (p.compress || p.act_sparsity) throw Unsupported("compressed / sparse convolutions are not implemented");
-        if (IC % 16 != 0) throw Unsupported("input channels not a multiple of 16 need the padded / compressed input path");
         const int64_t KY = p.weight.shape[2], KX = p.weight.shape[3];
         if (p.weight.shape[0] != OC || p.weight.shape[1] != IC) throw std::runtime_error("weight shape does not match input / output channels");
+        // Input channels that are no multiple of 16: the builder pads the input buffer and the weights' IC dimension to
+        // the alignment (paddedInputCMXShape / paddedWeightsCMXShape, buildZMConvTest.cpp:111-136). The descriptor
+        // describes those padded buffers; the caller fills the padding channels of the weights with the weights' zero
+        // point (so that they contribute nothing) and may leave any bytes in the padding channels of the input.
+        const int64_t ICP = (IC + 15) / 16 * 16;
+        if (ICP != IC) {
+            dense_nhwc(&d->input, p.input.dtype, N, ICP, IH, IW, p.input.zero_point);
+        }
         d->weights.dtype = p.weight.dtype;
         d->weights.zero_point = (int32_t)p.weight.zero_point;
         d->weights.dims[0] = OC;
-        d->weights.dims[1] = IC;
+        d->weights.dims[1] = ICP;
         d->weights.dims[2] = KY;
         d->weights.dims[3] = KX;
-        d->weights.strides_bytes[1] = 1;             // OYXI: IC innermost
-        d->weights.strides_bytes[3] = IC;            // KX
-        d->weights.strides_bytes[2] = IC * KX;       // KY
-        d->weights.strides_bytes[0] = IC * KX * KY;  // OC
+        d->weights.strides_bytes[1] = 1;              // OYXI: IC innermost
+        d->weights.strides_bytes[3] = ICP;            // KX
+        d->weights.strides_bytes[2] = ICP * KX;       // KY
+        d->weights.strides_bytes[0] = ICP * KX * KY;  // OC
         table_tensor(OC);
-        fill_table(p.arch, OC, IC * KX * KY, c.wt.scales, c.in.scales, c.out.scales, table);
+        fill_table(p.arch, OC, ICP * KX * KY, c.wt.scales, c.in.scales, c.out.scales, table);
         var->mpe_mode = p.mpe_mode;
         // storage-domain clamp, activation maximum, PReLU slope (buildZMConvTest.cpp:375-404)
         ppe->clamp_low = storage_min(out_dt);

@@ -3,6 +3,7 @@
 // reference's src/vpux_compiler/src/.
 #include <cfloat>
 #include <climits>
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 
@@ -259,6 +260,92 @@ nce_result_t ncePpeForEltwiseAdd(int32_t arch, nce_quant_t in1, nce_quant_t in2,
         ppe->quant_mult = static_cast<int32_t>(a.mult);
         ppe->quant_shift = a.shift;
         ppe->quant_post_shift = a.post_shift;
+    }
+    return NCE_RESULT_SUCCESS;
+}
+
+// Bits of a float converted to IEEE half / bfloat16 with round-to-nearest-even, sign-extended from 16 bits
+// (the reference reinterprets the 16-bit pattern as int16_t, fuse_clamp.cpp:54-57,63-66).
+static int32_t f16_bits(float v) {
+    uint32_t x;
+    memcpy(&x, &v, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const int32_t exp = static_cast<int32_t>((x >> 23) & 0xFF) - 127 + 15;
+    uint32_t man = x & 0x7FFFFFu;
+    uint32_t h;
+    if (((x >> 23) & 0xFF) == 0xFF) {
+        h = sign | 0x7C00u | (man ? 0x200u : 0u);
+    } else if (exp >= 31) {
+        h = sign | 0x7C00u;
+    } else if (exp <= 0) {
+        if (exp < -10) {
+            h = sign;
+        } else {
+            man |= 0x800000u;
+            const int shift = 14 - exp;  // 14..24
+            uint32_t r = man >> shift;
+            const uint32_t rem = man & ((1u << shift) - 1), half = 1u << (shift - 1);
+            if (rem > half || (rem == half && (r & 1))) ++r;
+            h = sign | r;
+        }
+    } else {
+        uint32_t r = (static_cast<uint32_t>(exp) << 10) | (man >> 13);
+        const uint32_t rem = man & 0x1FFFu;
+        if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) ++r;  // a carry into the exponent is the right result
+        h = sign | r;
+    }
+    return static_cast<int32_t>(static_cast<int16_t>(static_cast<uint16_t>(h)));
+}
+static int32_t bf16_bits(float v) {
+    uint32_t x;
+    memcpy(&x, &v, 4);
+    if ((x & 0x7F800000u) == 0x7F800000u && (x & 0x7FFFFFu)) return static_cast<int32_t>(static_cast<int16_t>(static_cast<uint16_t>((x >> 16) | 0x40u)));
+    const uint32_t r = x + 0x7FFFu + ((x >> 16) & 1u);
+    return static_cast<int32_t>(static_cast<int16_t>(static_cast<uint16_t>(r >> 16)));
+}
+
+nce_result_t ncePpeFuseClamp(nce_quant_t out, double clamp_min, double clamp_max, nce_ppe_task_t* ppe) {
+    if (!ppe) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    if (out.dtype == NCE_DT_U8 || out.dtype == NCE_DT_I8) {
+        if (out.scale == 0) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+        const double lo = std::round(clamp_min / out.scale) + out.zero_point;  // fuse_clamp.cpp:46-51
+        const double hi = std::round(clamp_max / out.scale) + out.zero_point;
+        // checked_cast<int32_t>: a value outside int32 is an error
+        if (!(lo >= static_cast<double>(INT32_MIN) && lo <= static_cast<double>(INT32_MAX) && hi >= static_cast<double>(INT32_MIN) &&
+              hi <= static_cast<double>(INT32_MAX)))
+            return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+        ppe->clamp_low = std::max(ppe->clamp_low, static_cast<int32_t>(lo));
+        ppe->clamp_high = std::min(ppe->clamp_high, static_cast<int32_t>(hi));
+        return NCE_RESULT_SUCCESS;  // the mode stays (getPPEMode, :74-78)
+    }
+    if (out.dtype == NCE_DT_F16 || out.dtype == NCE_DT_BF16) {
+        if (clamp_min != 0.0) return NCE_RESULT_ERROR_UNSUPPORTED;  // isLegalClamp: such a Clamp is not fused (:141-143)
+        const int32_t bits = out.dtype == NCE_DT_F16 ? f16_bits(static_cast<float>(clamp_max)) : bf16_bits(static_cast<float>(clamp_max));
+        ppe->clamp_low = INT32_MIN;
+        ppe->clamp_high = std::min(ppe->clamp_high, bits);
+        ppe->mode = NCE_PPE_LRELUX;  // :80-82
+        return NCE_RESULT_SUCCESS;
+    }
+    return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+}
+
+nce_result_t nceConvWeightSetBytes(int64_t ic, int64_t ky, int64_t kx, int64_t* set_bytes, int64_t* pad_bytes) {
+    if (!set_bytes || !pad_bytes || ic <= 0 || ky <= 0 || kx <= 0 || ic > (1 << 24) || ky > 1024 || kx > 1024) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    const int64_t n = ic * ky * kx;  // 8-bit elements
+    *set_bytes = (n + 15) / 16 * 16;
+    *pad_bytes = *set_bytes - n;
+    return NCE_RESULT_SUCCESS;
+}
+
+nce_result_t nceWeightsTableCheck(const int32_t* table, int32_t oc, int32_t weights_ptr_step) {
+    if (!table || oc <= 0 || weights_ptr_step < 0) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    if (weights_ptr_step % 16 != 0) return NCE_RESULT_ERROR_INVALID_ARGUMENT;  // nce_sparsity.cpp:399-412
+    const int64_t base = table[0];
+    if (base % 16 != 0) return NCE_RESULT_ERROR_INVALID_ARGUMENT;             // :504-506
+    for (int32_t c = 0; c < oc; ++c) {
+        const int32_t* row = table + 4 * static_cast<int64_t>(c);
+        if (static_cast<int64_t>(row[0]) - base != static_cast<int64_t>(c) * weights_ptr_step) return NCE_RESULT_ERROR_UNSUPPORTED;
+        if (row[1] != 0xFFFFFF) return NCE_RESULT_ERROR_UNSUPPORTED;           // a sparsity map: not on this path
     }
     return NCE_RESULT_SUCCESS;
 }

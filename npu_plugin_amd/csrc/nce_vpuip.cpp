@@ -149,6 +149,7 @@ struct TensorType {
     int64_t strides_elems[4] = {0, 0, 0, 0};
     int32_t section = -1, index = 0;
     bool plain_memref = false;  // false: distributed / sparse / unknown type
+    std::string type_name;      // the type as written when it is no plain memref; else the element type as written
 };
 
 struct Aliases {
@@ -257,7 +258,10 @@ TensorType parse_type(const std::string& text, const Aliases& al) {
         v = trim(it->second);
     }
     TensorType t;
-    if (!starts_with(v, 0, "memref<")) return t;  // distributed / sparse buffers: not a plain memref
+    if (!starts_with(v, 0, "memref<")) {  // distributed / sparse buffers: not a plain memref
+        t.type_name = v.substr(0, v.find_first_of("< "));
+        return t;
+    }
     t.plain_memref = true;
     const std::string body = inside(v, 6);
     const std::vector<std::string> parts = split_top(body);
@@ -274,6 +278,7 @@ TensorType parse_type(const std::string& text, const Aliases& al) {
         pos = e + 1;
     }
     parse_element(se.substr(pos), al, &t);
+    t.type_name = trim(se.substr(pos));
     for (int i = 0; i < 4; ++i) t.perm[i] = i;
     for (size_t i = 1; i < parts.size(); ++i) {
         const std::string& p = parts[i];
@@ -298,6 +303,8 @@ TensorType parse_type(const std::string& text, const Aliases& al) {
 struct Buffer {
     nce_vpuip_buffer_t pub{};
     bool plain = false;
+    bool dense = false;        // bytes are contiguous: byte_size == number of elements * element size
+    std::string type_name;     // see TensorType
 };
 
 struct Task {
@@ -338,8 +345,21 @@ int line_of(const std::string& s, size_t pos) {
     return 1 + (int)std::count(s.begin(), s.begin() + std::min(pos, s.size()), '\n');
 }
 
+// a * b and a + b for non-negative byte counts; a ParseError instead of a wrapped value
+int64_t mul_checked(int64_t a, int64_t b) {
+    int64_t r;
+    if (a < 0 || b < 0 || __builtin_mul_overflow(a, b, &r)) throw ParseError("tensor extent overflows 63 bits");
+    return r;
+}
+int64_t add_checked(int64_t a, int64_t b) {
+    int64_t r;
+    if (a < 0 || b < 0 || __builtin_add_overflow(a, b, &r)) throw ParseError("tensor extent overflows 63 bits");
+    return r;
+}
+
 void finish_buffer(const TensorType& t, Buffer* b) {
     b->plain = t.plain_memref;
+    b->type_name = t.type_name;
     b->pub.dtype = t.dtype;
     b->pub.elem_bytes = t.elem_bytes;
     b->pub.zero_point = t.zero_point;
@@ -349,14 +369,14 @@ void finish_buffer(const TensorType& t, Buffer* b) {
     for (int i = 0; i < t.rank; ++i) b->pub.dims[i + shift] = t.dims[i];
     int64_t strides[4] = {0, 0, 0, 0};
     if (t.has_strides) {
-        for (int i = 0; i < t.rank; ++i) strides[i + shift] = t.strides_elems[i] * t.elem_bytes;
+        for (int i = 0; i < t.rank; ++i) strides[i + shift] = mul_checked(t.strides_elems[i], t.elem_bytes);
     } else {
         int64_t s = t.elem_bytes;
         for (int i = t.rank - 1; i >= 0; --i) {
             const int d = t.perm[i];
             if (d < 0 || d >= t.rank) throw ParseError("layout names a dimension outside the rank");
             strides[d + shift] = s;
-            s *= t.dims[d];
+            s = mul_checked(s, t.dims[d]);
         }
     }
     int64_t span = t.elem_bytes;
@@ -365,8 +385,14 @@ void finish_buffer(const TensorType& t, Buffer* b) {
         b->pub.strides_bytes[i] = strides[i];
     }
     span = t.elem_bytes;
-    for (int i = 0; i < 4; ++i) span += (b->pub.dims[i] - 1) * b->pub.strides_bytes[i];
+    int64_t elems = 1;
+    for (int i = 0; i < 4; ++i) {
+        if (b->pub.dims[i] <= 0) throw ParseError("tensor with an empty dimension");
+        span = add_checked(span, mul_checked(b->pub.dims[i] - 1, b->pub.strides_bytes[i]));
+        elems = mul_checked(elems, b->pub.dims[i]);
+    }
     b->pub.byte_size = span;
+    b->dense = span == mul_checked(elems, t.elem_bytes);
 }
 
 int add_buffer(nce_vpuip_program_s* p, const std::string& name, const TensorType& t, int32_t section, int32_t index, int64_t offset) {
@@ -377,6 +403,7 @@ int add_buffer(nce_vpuip_program_s* p, const std::string& name, const TensorType
     b.pub.section = section;
     b.pub.index = index;
     b.pub.byte_offset = offset;
+    add_checked(offset, b.pub.byte_size);  // (the end of the buffer inside its section must be representable)
     p->buffers.push_back(b);
     p->by_name[name] = (int)p->buffers.size() - 1;
     return (int)p->buffers.size() - 1;
@@ -609,8 +636,15 @@ size_t parse_nce_task(nce_vpuip_program_s* p, const std::string& s, size_t pos, 
     set_tensor(&d.output, p->buffers[task.output]);
     if (task.weights >= 0) set_tensor(&d.weights, p->buffers[task.weights]);
     if (task.table >= 0) set_tensor(&d.weight_table, p->buffers[task.table]);
-    for (const int b : {task.input, task.output, task.weights, task.table})
-        if (b >= 0 && !p->buffers[b].plain) throw ParseError(where + "operand " + p->buffers[b].pub.name + " is not a plain memref (distributed / sparse buffers are not supported)");
+    for (const int b : {task.input, task.output, task.weights, task.table}) {
+        if (b < 0) continue;
+        const Buffer& buf = p->buffers[b];
+        if (!buf.plain)
+            throw ParseError(where + "operand " + buf.pub.name + " has type " + (buf.type_name.empty() ? "(unknown)" : buf.type_name) +
+                             ": only plain memrefs are supported (no distributed or sparse buffers)");
+        if (buf.pub.dtype < 0)
+            throw ParseError(where + "operand " + buf.pub.name + " has element type " + buf.type_name + ": only u8 / i8 tensors and si32 tables are executable here");
+    }
     Op op;
     op.kind = NCE_VPUIP_OP_NCE_TASK;
     op.task = (int)p->tasks.size();
@@ -701,12 +735,27 @@ void parse_program(const std::string& raw, nce_vpuip_program_s* p) {
         const TensorType t = parse_type(a.substr(colon + 1), al);
         add_buffer(p, trim(a.substr(0, colon)), t, NCE_VPUIP_SECTION_ARGUMENT, argno++, 0);
     }
+    // The body of THIS function: from the first '{' outside the signature's types to its matching '}'. SSA names and
+    // operations of later functions of the module (lit files hold several) are not part of the program.
+    size_t body_open = std::string::npos;
+    {
+        int depth = 0;
+        for (size_t i = rp + 1; i < s.size(); ++i) {
+            const char c = s[i];
+            if (c == '-' && i + 1 < s.size() && s[i + 1] == '>') { ++i; continue; }
+            if (c == '{' && depth == 0) { body_open = i; break; }
+            if (c == '<' || c == '(' || c == '[' || c == '{') ++depth;
+            else if (c == '>' || c == ')' || c == ']' || c == '}') --depth;
+        }
+    }
+    if (body_open == std::string::npos) throw ParseError("function @" + p->function + " has no body");
+    const size_t body_close = balanced_end(s, body_open + 1);
     // body: the three operation kinds, in text order
-    size_t pos = rp;
+    size_t pos = body_open;
     for (;;) {
         const size_t db = s.find("VPURT.DeclareBuffer", pos), nt = s.find("VPUIP.NCEClusterTask", pos), dm = s.find("VPUIP.NNDMA", pos);
         const size_t next = std::min(db, std::min(nt, dm));
-        if (next == std::string::npos) break;
+        if (next == std::string::npos || next >= body_close) break;
         if (next == db) {
             const int line = line_of(s, db);
             const std::string name = result_name_before(s, db);
@@ -864,29 +913,38 @@ nce_result_t nceVpuipGetTask(nce_vpuip_program_handle_t program, int32_t task_in
 nce_result_t nceVpuipEnqueue(nce_vpuip_program_handle_t program, nce_executor_handle_t executor, void* hip_stream) {
     if (program == nullptr || executor == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
     // the executor's log is not reachable from here; errors of the tasks themselves land in it through Enqueue
-    for (const Op& op : program->ops) {
-        if (op.kind == NCE_VPUIP_OP_NCE_TASK) {
-            nce_cluster_task_desc_t d;
-            nce_result_t r = resolve_task(program, op.task, &d, nullptr);
-            if (r != NCE_RESULT_SUCCESS) return r;
-            r = nceClusterTaskEnqueue(executor, &d, hip_stream);
-            if (r != NCE_RESULT_SUCCESS) return r;
-        } else {
-            if (op.src < 0 || op.dst < 0) return NCE_RESULT_ERROR_UNSUPPORTED;  // e.g. a copy out of a constant
-            const Buffer& a = program->buffers[op.src];
-            const Buffer& b = program->buffers[op.dst];
-            if (a.pub.byte_size != b.pub.byte_size || a.pub.elem_bytes != b.pub.elem_bytes ||
-                memcmp(a.pub.dims, b.pub.dims, sizeof(a.pub.dims)) != 0 || memcmp(a.pub.strides_bytes, b.pub.strides_bytes, sizeof(a.pub.strides_bytes)) != 0)
-                return NCE_RESULT_ERROR_UNSUPPORTED;  // layout-changing DMAs are not implemented
-            std::string why;
-            uint8_t* src = address_of(program, a, &why);
-            uint8_t* dst = address_of(program, b, &why);
-            if (src == nullptr || dst == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
-            if (hipMemcpyAsync(dst, src, (size_t)a.pub.byte_size, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(hip_stream)) != hipSuccess)
-                return NCE_RESULT_ERROR_UNKNOWN;
+    try {
+        for (const Op& op : program->ops) {
+            if (op.kind == NCE_VPUIP_OP_NCE_TASK) {
+                nce_cluster_task_desc_t d;
+                nce_result_t r = resolve_task(program, op.task, &d, nullptr);
+                if (r != NCE_RESULT_SUCCESS) return r;
+                r = nceClusterTaskEnqueue(executor, &d, hip_stream);  // (sets the executor's device)
+                if (r != NCE_RESULT_SUCCESS) return r;
+            } else {
+                if (op.src < 0 || op.dst < 0) return NCE_RESULT_ERROR_UNSUPPORTED;  // e.g. a copy out of a constant
+                const Buffer& a = program->buffers[op.src];
+                const Buffer& b = program->buffers[op.dst];
+                // One flat copy: both sides dense (a strided view would also overwrite the bytes between its rows) and of
+                // the same shape and order; layout-changing and strided DMAs are not implemented.
+                if (!a.dense || !b.dense || a.pub.byte_size != b.pub.byte_size || a.pub.elem_bytes != b.pub.elem_bytes ||
+                    memcmp(a.pub.dims, b.pub.dims, sizeof(a.pub.dims)) != 0 || memcmp(a.pub.strides_bytes, b.pub.strides_bytes, sizeof(a.pub.strides_bytes)) != 0)
+                    return NCE_RESULT_ERROR_UNSUPPORTED;
+                std::string why;
+                uint8_t* src = address_of(program, a, &why);
+                uint8_t* dst = address_of(program, b, &why);
+                if (src == nullptr || dst == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+                // (the copy goes to the device the stream belongs to; a task before it has made the executor's device current)
+                if (hipMemcpyAsync(dst, src, (size_t)a.pub.byte_size, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(hip_stream)) != hipSuccess)
+                    return NCE_RESULT_ERROR_UNKNOWN;
+            }
         }
+        return NCE_RESULT_SUCCESS;
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (...) {
+        return NCE_RESULT_ERROR_UNKNOWN;
     }
-    return NCE_RESULT_SUCCESS;
 }
 
 }  // extern "C"

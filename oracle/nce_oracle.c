@@ -185,6 +185,19 @@ int nce_oracle_ppe_stage1(int arch, int postop, double a0, double a1, int32_t st
     }
 }
 
+/* fuse_clamp.cpp:34-53: quantized bounds round(min / scale) + zp and round(max / scale) + zp (std::round: halves away
+ * from zero), intersected with the range the op's PPE already has. */
+int nce_oracle_fuse_clamp_quant(double out_scale, int32_t out_zp, double clamp_min, double clamp_max, int32_t* clamp_low,
+                                int32_t* clamp_high) {
+    if (out_scale == 0.0 || !clamp_low || !clamp_high) return -1;
+    const double qlo = round(clamp_min / out_scale) + (double)out_zp;
+    const double qhi = round(clamp_max / out_scale) + (double)out_zp;
+    if (qlo < -2147483648.0 || qlo > 2147483647.0 || qhi < -2147483648.0 || qhi > 2147483647.0) return -1;
+    if ((int32_t)qlo > *clamp_low) *clamp_low = (int32_t)qlo;
+    if ((int32_t)qhi < *clamp_high) *clamp_high = (int32_t)qhi;
+    return 0;
+}
+
 /* dialect/VPU/transforms/passes/setup_ppe.cpp:12-33 (mode) and :123-195 (clamps), quantized output */
 void nce_oracle_ppe_stage2_37xx(int has_ppe, int32_t storage_min, int32_t storage_max, int32_t out_zp,
                                 nce_ppe_task_t* ppe) {

@@ -81,6 +81,12 @@ int nce_oracle_ppe_stage1(int arch, int postop, double a0, double a1, int32_t st
 void nce_oracle_ppe_stage2_37xx(int has_ppe, int32_t storage_min, int32_t storage_max, int32_t out_zp,
                                 nce_ppe_task_t* ppe);
 
+/* FuseClamp for a quantized (per-tensor) output: ClampConverter::getTargetClamps,
+ * src/vpux_compiler/src/dialect/VPU/transforms/passes/fuse_clamp.cpp:34-53. Rewrites *clamp_low / *clamp_high (the
+ * op's PPE range on entry). The mode does not change for quantized outputs (:74-78). Returns 0 / -1. */
+int nce_oracle_fuse_clamp_quant(double out_scale, int32_t out_zp, double clamp_min, double clamp_max, int32_t* clamp_low,
+                                int32_t* clamp_high);
+
 /* ---- per-element integer pipeline ---------------------------------------------------------- */
 
 int64_t nce_oracle_rshift_round(int64_t p, int32_t shift, int32_t round_mode);

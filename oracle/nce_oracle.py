@@ -41,6 +41,7 @@ def lib():
                                             C.c_int32, _P(abi.PpeTask)]
         L.nce_oracle_ppe_stage2_37xx.argtypes = [C.c_int, C.c_int32, C.c_int32, C.c_int32, _P(abi.PpeTask)]
         L.nce_oracle_ppe_stage2_37xx.restype = None
+        L.nce_oracle_fuse_clamp_quant.argtypes = [C.c_double, C.c_int32, C.c_double, C.c_double, _P(C.c_int32), _P(C.c_int32)]
         L.nce_oracle_rshift_round.argtypes = [C.c_int64, C.c_int32, C.c_int32]
         L.nce_oracle_rshift_round.restype = C.c_int64
         L.nce_oracle_ppe.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P(abi.PpeTask), C.c_int32, C.c_int32]

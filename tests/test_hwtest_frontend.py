@@ -66,6 +66,13 @@ def test_parse_errors_carry_the_reference_messages(mutate, message):
     assert e.value.code == abi.ERROR_INVALID_ARGUMENT and message in e.value.log
 
 
+def test_deeply_nested_json_is_a_parse_error_not_a_crash():
+    for text in ("[" * 100000, '{"a":' * 5000 + "1" + "}" * 5000, '{"input": ' + "[" * 70 + "]" * 70 + "}"):
+        with pytest.raises(nce.NCEError) as e:
+            hwtest.parse(text)
+        assert e.value.code == abi.ERROR_INVALID_ARGUMENT and "nesting" in e.value.log
+
+
 def test_comment_lines_names_and_other_case_types():
     text = "// RUN: vpux-translate --import-HWTEST %s\n   // second comment\n" + load("zmajor_conv_u8.json")
     case = hwtest.parse(text)
@@ -93,6 +100,8 @@ def buffers(case, rng):
     i, w, o = case.info.input, case.info.weight, case.info.output
     n, c, h, wd = i.shape
     x = rng.integers(0, 256, (n, h, wd, c), dtype=np.uint8)
+    if case.task_type == abi.TASK_CONV and c % 16 != 0:
+        return padded_conv_buffers(case, rng, x)
     extent = {"n": o.shape[0], "c": o.shape[1], "h": o.shape[2], "w": o.shape[3]}
     out = np.zeros([extent[d] for d in case.output_order], dtype=np.uint8)   # dense in the case's output order
     wt = None
@@ -106,6 +115,58 @@ def buffers(case, rng):
     elif case.task_type == abi.TASK_ELTWISE:
         wt = rng.integers(0, 256, x.shape, dtype=np.uint8)
     return x, wt, out
+
+
+def padded_conv_buffers(case, rng, x):
+    """Input channels that are no multiple of 16: the buffers the builder allocates (channels rounded up to 16). The
+    padding channels of the weights hold the weights' zero point; those of the input hold noise."""
+    i, w, o = case.info.input, case.info.weight, case.info.output
+    n, c, h, wd = i.shape
+    cp = (c + 15) // 16 * 16
+    xp = rng.integers(0, 256, (n, h, wd, cp), dtype=np.uint8)
+    xp[..., :c] = x
+    dt = np.int8 if w.dtype == abi.DT_I8 else np.uint8
+    wt = np.full((w.shape[0], w.shape[2], w.shape[3], cp), w.zero_point, dtype=dt)
+    wt[..., :c] = rng.integers(-127 if dt == np.int8 else 0, 128 if dt == np.int8 else 256, (w.shape[0], w.shape[2], w.shape[3], c)).astype(dt)
+    out = np.zeros((o.shape[0], o.shape[2], o.shape[3], o.shape[1]), dtype=np.uint8)
+    return xp, wt, out
+
+
+def test_zmajor_conv_with_three_input_channels_is_padded_like_the_builder(validator):
+    """IC = 3: descriptor over 16-channel buffers (buildZMConvTest.cpp:111-136); the result equals an IC = 3 convolution
+    computed directly in integers, whatever the padding channels of the input hold."""
+    from oracle import nce_oracle
+    case = hwtest.parse(load("zmajor_conv3x3_ic3_padded.json"))
+    rng = np.random.default_rng(5)
+    x, wt, out = buffers(case, rng)
+    task = case.build_task(x, wt, out)
+    d = task.desc
+    assert list(d.input.dims) == [1, 16, 20, 20] and list(d.weights.dims) == [32, 16, 3, 3]
+    assert list(d.weights.strides_bytes) == [144, 1, 48, 16] and task.table[1][0] - task.table[0][0] == 144
+    validator.validate(task)
+    nce_oracle.run(task)
+    x2 = x.copy()
+    x2[..., 3:] = rng.integers(0, 256, x2[..., 3:].shape, dtype=np.uint8)   # other noise in the padding: same bytes out
+    out2 = np.zeros_like(out)
+    nce_oracle.run(case.build_task(x2, wt, out2))
+    assert out.std() > 1.0 and np.array_equal(out, out2)
+    # direct integer evaluation over the three real channels at one interior and one corner pixel
+    zp_a, zp_w = case.info.input.zero_point, case.info.weight.zero_point
+    for (oy, ox) in ((7, 9), (0, 0)):
+        for oc in (0, 31):
+            acc = 0
+            for ky in range(3):
+                for kx in range(3):
+                    iy, ix = oy + ky - 1, ox + kx - 1
+                    if 0 <= iy < 20 and 0 <= ix < 20:
+                        acc += int(((x[0, iy, ix, :3].astype(np.int64) - zp_a) * (wt[oc, ky, kx, :3].astype(np.int64) - zp_w)).sum())
+            w2 = int(task.table[oc][2]) & 0xFFFFFFFF
+            mult, shift = w2 >> 16, (w2 >> 8) & 0x3F
+            y = (acc * mult + (1 << (shift - 1))) >> shift
+            if y < 0:
+                y = (y * task._ppe.lrelu_mult + ((1 << (task._ppe.lrelu_shift - 1)) if task._ppe.lrelu_shift else 0)) >> task._ppe.lrelu_shift
+            y = min(max(y + case.info.output.zero_point, task._ppe.clamp_low), task._ppe.clamp_high)
+            assert out[0, oy, ox, oc] == y, (oy, ox, oc)
 
 
 def test_zmajor_conv_descriptor_follows_the_builder(validator):
@@ -222,7 +283,7 @@ def test_output_order_becomes_output_strides(validator):
     assert ref.std() > 1.0 and np.array_equal(out.transpose(0, 2, 3, 1), ref)
 
 
-ALL = ["zmajor_conv_u8.json", "zmajor_conv3x3_lrelu_per_channel.json", "zmajor_conv3x3_output_nchw.json", "depthwise_u8.json", "maxpool_u8.json",
+ALL = ["zmajor_conv_u8.json", "zmajor_conv3x3_ic3_padded.json", "zmajor_conv3x3_lrelu_per_channel.json", "zmajor_conv3x3_output_nchw.json", "depthwise_u8.json", "maxpool_u8.json",
        "avgpool_u8.json", "avgpool_u8_per_channel.json", "eltwise_add_u8.json"]
 
 

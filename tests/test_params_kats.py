@@ -5,6 +5,7 @@ import ctypes as C
 import json
 import os
 
+import numpy as np
 import pytest
 
 from npu_plugin_amd import _abi as abi
@@ -185,3 +186,105 @@ def test_avgpool_and_eltwise_ppe_generators():
                                    abi.Quant(1.0, 3, abi.DT_U8), abi.POSTOP_NONE, 0, 0, C.byref(p)) == abi.SUCCESS
     assert (p.mode, p.has_in_mult, p.quant_mult, p.quant_shift, p.clamp_low, p.clamp_high, p.clamp_domain) == \
         (abi.PPE_ADD, 0, 16384, 14, -3, 252, abi.CLAMP_PRE_ZP)
+
+
+DTYPES = {"u8": abi.DT_U8, "i8": abi.DT_I8, "f16": abi.DT_F16, "bf16": abi.DT_BF16}
+
+
+@pytest.mark.parametrize("k", KATS["fuse_clamp_37xx"], ids=lambda k: k["name"])
+def test_fuse_clamp_lit_cases(k):
+    """ncePpeFuseClamp (and the oracle's quantized twin) against the before / after PPE attributes of the reference's
+    fuse_clamp lit file."""
+    lib = abi.load_library()
+    p = abi.PpeTask()
+    p.mode, p.clamp_low, p.clamp_high, p.lrelu_mult, p.lrelu_shift = MODES[k["in"]["mode"]], k["in"]["low"], k["in"]["high"], 1024, 13
+    rc = lib.ncePpeFuseClamp(abi.Quant(k["scale"], k["zp"], DTYPES[k["dtype"]]), k["min"], k["max"], C.byref(p))
+    if k["out"] is None:
+        assert rc == abi.ERROR_UNSUPPORTED
+        assert (p.mode, p.clamp_low, p.clamp_high) == (MODES[k["in"]["mode"]], k["in"]["low"], k["in"]["high"])
+        return
+    assert rc == abi.SUCCESS
+    assert (p.mode, p.clamp_low, p.clamp_high, p.lrelu_mult, p.lrelu_shift) == (MODES[k["out"]["mode"]], k["out"]["low"], k["out"]["high"], 1024, 13)
+    if k["dtype"] in ("u8", "i8"):
+        lo, hi = C.c_int32(k["in"]["low"]), C.c_int32(k["in"]["high"])
+        assert O.lib().nce_oracle_fuse_clamp_quant(k["scale"], k["zp"], k["min"], k["max"], C.byref(lo), C.byref(hi)) == 0
+        assert (lo.value, hi.value) == (k["out"]["low"], k["out"]["high"])
+
+
+def test_fuse_clamp_float_bits_and_errors():
+    """Half and bfloat16 bit patterns against numpy / exact powers of two; range errors."""
+    lib = abi.load_library()
+    for v in [0.0, 1.0, 6.0, 120.0, 128.0, 65504.0, 1e-3, 0.333251953125, 5.960464477539063e-08, 70000.0, 2049.0, 2051.0]:
+        p = abi.PpeTask()
+        p.clamp_low, p.clamp_high = -2**31, 2**31 - 1
+        assert lib.ncePpeFuseClamp(abi.Quant(1.0, 0, abi.DT_F16), 0.0, v, C.byref(p)) == abi.SUCCESS
+        with np.errstate(over="ignore"):
+            assert p.clamp_high == int(np.array([v], dtype=np.float32).astype(np.float16).view(np.int16)[0]), v
+        assert (p.clamp_low, p.mode) == (-2**31, abi.PPE_LRELUX)
+    for v, bits in [(1.0, 0x3F80), (128.0, 0x4300), (6.0, 0x40C0), (1.00390625, 0x3F80), (1.01171875, 0x3F82)]:  # ties to even
+        p = abi.PpeTask()
+        p.clamp_low, p.clamp_high = -2**31, 2**31 - 1
+        assert lib.ncePpeFuseClamp(abi.Quant(1.0, 0, abi.DT_BF16), 0.0, v, C.byref(p)) == abi.SUCCESS
+        assert p.clamp_high == bits, v
+    p = abi.PpeTask()
+    assert lib.ncePpeFuseClamp(abi.Quant(1e-12, 0, abi.DT_U8), 0.0, 1e3, C.byref(p)) == abi.ERROR_INVALID_ARGUMENT  # beyond int32
+    assert lib.ncePpeFuseClamp(abi.Quant(0.0, 0, abi.DT_U8), 0.0, 1.0, C.byref(p)) == abi.ERROR_INVALID_ARGUMENT
+    assert lib.ncePpeFuseClamp(abi.Quant(1.0, 0, abi.DT_SI32), 0.0, 1.0, C.byref(p)) == abi.ERROR_INVALID_ARGUMENT
+
+
+def test_weight_set_padding_layout():
+    lib = abi.load_library()
+    for k in KATS["weights_zero_pad"]:
+        sb, pb = C.c_int64(), C.c_int64()
+        assert lib.nceConvWeightSetBytes(k["ic"], k["ky"], k["kx"], C.byref(sb), C.byref(pb)) == abi.SUCCESS
+        assert [k["oc"], 1, 1, sb.value] == k["padded_shape"] and pb.value == k["pad"]
+    sb, pb = C.c_int64(), C.c_int64()
+    assert lib.nceConvWeightSetBytes(64, 3, 3, C.byref(sb), C.byref(pb)) == abi.SUCCESS and (sb.value, pb.value) == (576, 0)
+    assert lib.nceConvWeightSetBytes(0, 3, 3, C.byref(sb), C.byref(pb)) == abi.ERROR_INVALID_ARGUMENT
+
+
+def test_weights_table_pointer_contract():
+    """Words [0] and [1]: the generator's tables pass; re-ordered pointers, a misaligned step and a sparsity pointer do not."""
+    lib = abi.load_library()
+    oc = 8
+    t = (C.c_int32 * (4 * oc))()
+    ws = (C.c_double * 1)(0.01)
+    assert lib.nceWeightsTableFill(1, oc, 4096, 576, 0xFFFFFF, 0.02, 0.05, ws, 1, None, t) == abi.SUCCESS
+    assert lib.nceWeightsTableCheck(t, oc, 576) == abi.SUCCESS
+    t[4 * 3], t[4 * 4] = t[4 * 4], t[4 * 3]
+    assert lib.nceWeightsTableCheck(t, oc, 576) == abi.ERROR_UNSUPPORTED
+    t[4 * 3], t[4 * 4] = t[4 * 4], t[4 * 3]
+    t[4 * 2 + 1] = 1024
+    assert lib.nceWeightsTableCheck(t, oc, 576) == abi.ERROR_UNSUPPORTED
+    t[4 * 2 + 1] = 0xFFFFFF
+    assert lib.nceWeightsTableCheck(t, oc, 568) == abi.ERROR_INVALID_ARGUMENT
+    assert lib.nceWeightsTableCheck(t, oc, 592) == abi.ERROR_UNSUPPORTED
+
+
+def test_ppe_register_field_widths(validator):
+    """The validator accepts every PPE field at the largest value its register field holds (the masks of the reference's
+    register-map unit test) and rejects the next value."""
+    import npu_plugin_amd as nce
+    from tests import cases as K
+    m = KATS["ppe_register_field_masks_37xx"]
+
+    def rc(case):
+        task = K.build_task(case, case.input, case.weights, case.table, np.zeros(case.out_shape, dtype=np.uint8))
+        return validator.validate_code(task)
+
+    ok = lambda **ppe: K.conv_case(1, 1, 4, 4, 16, 16, ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=255, **ppe))
+    assert rc(ok(lrelu_mult=m["ppe_prelu_mult"], lrelu_shift=m["ppe_prelu_shift"])) == abi.SUCCESS
+    assert rc(ok(lrelu_mult=m["ppe_prelu_mult"] + 1, lrelu_shift=0)) == abi.ERROR_INVALID_ARGUMENT
+    assert rc(ok(lrelu_mult=1, lrelu_shift=m["ppe_prelu_shift"] + 1)) == abi.ERROR_INVALID_ARGUMENT
+    e = lambda **kw: K.eltwise_case(2, 1, 4, 4, 16, **kw)
+    assert rc(e(mult=m["ppe_scale_mult"], shift=m["ppe_scale_shift"], in1_mult=m["elop_scale_a"], in2_mult=m["elop_scale_b"])) == abi.SUCCESS
+    assert rc(e(mult=m["ppe_scale_mult"] + 1)) == abi.ERROR_INVALID_ARGUMENT
+    assert rc(e(shift=m["ppe_scale_shift"] + 1)) == abi.ERROR_INVALID_ARGUMENT
+    assert rc(e(in1_mult=m["elop_scale_a"] + 1)) == abi.ERROR_INVALID_ARGUMENT
+    assert rc(e(in2_mult=m["elop_scale_b"] + 1)) == abi.ERROR_INVALID_ARGUMENT
+    assert rc(e(ppe_extra=dict(round_mode=m["ppe_scale_round"]))) == abi.ERROR_INVALID_ARGUMENT  # three modes: 0..2
+    # the 9-bit zero-point register holds every u8 and i8 zero point
+    assert m["ppe_g8_bias_c"] >= 255 and -(m["ppe_g8_bias_c"] + 1) // 2 <= -128
+    # table word [2]: shift in 6 bits at bit 8, multiplier in 16 bits at bit 16
+    w = O.lib().nce_oracle_scale_word(1, m["ppe_scale_shift"], m["ppe_scale_mult"], 1) & 0xFFFFFFFF
+    assert w == (m["ppe_scale_mult"] << 16) | (m["ppe_scale_shift"] << 8)

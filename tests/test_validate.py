@@ -222,3 +222,26 @@ def test_executor_create_without_gpu_fails_loudly_when_a_device_is_requested():
     with pytest.raises(nce.NCEError) as e:
         nce.Executor(device_id=0, log_level=0)
     assert e.value.code == abi.ERROR_UNSUPPORTED
+
+
+def test_input_views_must_be_ordered_and_free_of_overlap(validator):
+    """Inputs get the same ordered, non-overlapping stride rule as outputs: rows that overlap pixels, images that
+    overlap rows and spans beyond the size cap are rejected; genuine sub-views (larger strides) stay legal."""
+    c = K.conv_case(1, 2, 6, 6, 16, 16)
+    t = task_of(c)
+    t.finalize()
+    assert validator.validate_code(t) == abi.SUCCESS
+    base = list(t.desc.input.strides_bytes)           # N, C, H, W = 576, 1, 96, 16
+
+    def with_strides(n, h, w):
+        t.desc.input.strides_bytes[0], t.desc.input.strides_bytes[2], t.desc.input.strides_bytes[3] = n, h, w
+        rc = validator.validate_code(t)
+        validator.log()
+        return rc
+
+    assert with_strides(1152, 192, 32) == abi.SUCCESS                   # a sub-view of a larger tensor
+    assert with_strides(576, 32, 16) == abi.ERROR_INVALID_ARGUMENT       # rows 32 bytes apart hold 6 pixels of 16 bytes
+    assert with_strides(96, 96, 16) == abi.ERROR_INVALID_ARGUMENT        # images one row apart
+    assert with_strides(576, 96, 0) == abi.ERROR_INVALID_ARGUMENT        # pixels on top of each other
+    assert with_strides(1 << 40, 96, 16) == abi.ERROR_INVALID_ARGUMENT   # span beyond the size cap
+    assert with_strides(*[base[0], base[2], base[3]]) == abi.SUCCESS

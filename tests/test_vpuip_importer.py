@@ -146,3 +146,107 @@ def test_program_runs_bit_exact(executor):
     mid, out = _reference_result(x, wt, table)
     assert np.array_equal(cmx[14336:18944].cpu().numpy().reshape(mid.shape), mid)
     assert np.array_equal(dout.cpu().numpy(), out)
+
+
+# ---- several functions in one module; the reference's own lit inputs where the reference tree is at hand ---------
+
+TWO_FUNCTIONS = TEXT + """
+
+func.func @second(%arg0: memref<1x16x4x4xf16, #NHWC, @DDR>) -> memref<1x16x4x4xf16, #NHWC, @DDR> {
+    %5 = VPURT.DeclareBuffer <CMX_NN> [0] <0> -> !VPUIP.DistributedBuffer<1x16x4x4xf16, #NHWC, @CMX_NN, {mode = "SEGMENTED", num_tiles = [1, 1, 2, 1], num_clusters = 2}>
+    VPURT.Task {
+        VPUIP.NNDMA inputs(%arg0 : memref<1x16x4x4xf16, #NHWC, @DDR>) outputs(%5 : !VPUIP.DistributedBuffer<1x16x4x4xf16, #NHWC, @CMX_NN, {mode = "SEGMENTED", num_tiles = [1, 1, 2, 1], num_clusters = 2}>) -> !VPUIP.DistributedBuffer<1x16x4x4xf16, #NHWC, @CMX_NN, {mode = "SEGMENTED", num_tiles = [1, 1, 2, 1], num_clusters = 2}>
+    }
+    return %arg0 : memref<1x16x4x4xf16, #NHWC, @DDR>
+}
+"""
+
+
+def test_only_the_first_function_is_the_program():
+    """SSA names are scoped per function: a later function that re-uses %5 for a distributed buffer neither adds
+    operations to the program nor changes what %5 means in the first one."""
+    one, two = vpuip.parse(TEXT), vpuip.parse(TWO_FUNCTIONS)
+    assert two.function == one.function and two.num_tasks == one.num_tasks and two.num_dmas == one.num_dmas
+    assert two.ops == one.ops
+    a, b = one.buffer("%5"), two.buffer("%5")
+    assert (a.section, a.byte_offset, a.byte_size, a.dtype) == (b.section, b.byte_offset, b.byte_size, b.dtype)
+
+
+def test_unsupported_operands_are_reported_by_their_real_reason():
+    text = """
+#NHWC = affine_map<(d0, d1, d2, d3) -> (d0, d2, d3, d1)>
+func.func @f(%arg0: memref<1x16x8x8xf16, #NHWC, @DDR>) -> memref<1x16x8x8xf16, #NHWC, @DDR> {
+    %0 = VPURT.DeclareBuffer <CMX_NN> [0] <0> -> memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>
+    %1 = VPURT.DeclareBuffer <CMX_NN> [0] <2048> -> memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>
+    VPURT.Task {
+      VPUIP.NCEClusterTask {kernel_padding = #VPU.Padding<left = 0 : i64, right = 0 : i64, top = 0 : i64, bottom = 0 : i64>, kernel_size = [1, 1], kernel_strides = [1, 1], task_type = #VPUIP.nce_task_type<MAXPOOL>}
+        input(%0 : memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>) parent_input(%0 : memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>)
+        parent_output(%1 : memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>) outputs(%1 : memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>)
+        -> memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]> variants : {
+          DPUTask {outStart = [0, 0, 0], outEnd = [7, 7, 15], mpe_mode = #VPU.mpe_mode<CUBOID_16x16>, pad = #VPU.Padding<left = 0 : i64, right = 0 : i64, top = 0 : i64, bottom = 0 : i64>}
+        } PPE : {
+        }
+    }
+    return %arg0 : memref<1x16x8x8xf16, #NHWC, @DDR>
+}
+"""
+    with pytest.raises(nce.NCEError) as e:
+        vpuip.parse(text)
+    assert "element type f16" in e.value.log, e.value.log
+    dist = text.replace("-> memref<1x16x8x8xf16, #NHWC, [@CMX_NN, 0]>\n    %1", "-> !VPUIP.DistributedBuffer<1x16x8x8xf16, #NHWC, @CMX_NN, {mode = \"DUPLICATED\", num_clusters = 2}>\n    %1", 1)
+    assert dist != text
+    with pytest.raises(nce.NCEError) as e:
+        vpuip.parse(dist)
+    assert "!VPUIP.DistributedBuffer" in e.value.log and "plain memref" in e.value.log, e.value.log
+
+
+REF_LIT = "/root/reference/tests/lit/NPU/conversion/passes/VPUIP2VPUMI37XX"
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_LIT), reason="the reference tree is not on this machine")
+def test_reference_lit_programs_read_in_place(validator):
+    """The reference's own VPUIP lit inputs, read where they lie: the u8 eltwise program parses into one task with the
+    attributes its text holds and validates; the fp16 max pool and convolution files are declined because of their
+    element type (each holds one function per split)."""
+    prog = vpuip.parse(open(os.path.join(REF_LIT, "nce_eltwise_37XX.mlir")).read())
+    assert prog.function == "singleEltwise" and prog.num_tasks == 1 and prog.num_dmas == 0
+    cmx = np.zeros(prog.section_size(vpuip.CMX_NN, 0), dtype=np.uint8)
+    prog.bind(vpuip.CMX_NN, 0, cmx)
+    d = prog.task(0).desc
+    p = d.ppe.contents
+    assert d.task_type == abi.TASK_ELTWISE and list(d.input.dims) == [1, 32, 56, 56] and list(d.input.strides_bytes) == [100352, 1, 1792, 32]
+    assert (p.mode, p.clamp_low, p.clamp_high, p.has_quant, p.quant_mult, p.quant_shift, p.has_in_mult) == (abi.PPE_ADD, 0, 255, 1, 16384, 14, 0)
+    assert d.num_variants == 1 and list(d.variants[0].out_end) == [55, 55, 31] and d.variants[0].mpe_mode == abi.MPE_CUBOID_8x16
+    assert d.input.data == cmx.ctypes.data + 100352 and d.weights.data == cmx.ctypes.data + 200704 and d.output.data == cmx.ctypes.data
+    validator.validate(prog.task(0))
+    for name in ("nce_maxpool_37XX.mlir", "nce_conv_37XX.mlir"):
+        with pytest.raises(nce.NCEError) as e:
+            vpuip.parse(open(os.path.join(REF_LIT, name)).read())
+        assert "element type f16" in e.value.log, e.value.log
+
+
+def test_strided_dma_is_declined_and_huge_extents_do_not_wrap(validator):
+    """A DMA between strided views is not run as one flat copy (it would overwrite the bytes between the rows), and
+    extents whose byte count leaves 63 bits are a parse error, not a wrapped size."""
+    strided = """
+#NHWC = affine_map<(d0, d1, d2, d3) -> (d0, d2, d3, d1)>
+func.func @f(%arg0: memref<1x16x8x8xui8, #NHWC, @DDR>) -> memref<1x16x8x8xui8, #NHWC, @DDR> {
+    %0 = VPURT.DeclareBuffer <DDR> <0> -> memref<1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}, @DDR>
+    %1 = VPURT.DeclareBuffer <DDR> <4096> -> memref<1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}, @DDR>
+    VPURT.Task {
+      VPUIP.NNDMA inputs(%0 : memref<1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}, @DDR>) outputs(%1 : memref<1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}, @DDR>) -> memref<1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}, @DDR>
+    }
+    return %arg0 : memref<1x16x8x8xui8, #NHWC, @DDR>
+}
+"""
+    prog = vpuip.parse(strided)
+    assert prog.num_dmas == 1
+    ddr = np.zeros(prog.section_size(vpuip.DDR, 0), dtype=np.uint8)
+    prog.bind(vpuip.DDR, 0, ddr)
+    with pytest.raises(nce.NCEError) as e:
+        prog.enqueue(validator)
+    assert e.value.code == abi.ERROR_UNSUPPORTED
+    huge = strided.replace("1x16x8x4xui8, {order = #NHWC, strides = [1024, 1, 128, 16]}", "4294967296x4294967296x8x4xui8, {order = #NHWC}")
+    with pytest.raises(nce.NCEError) as e:
+        vpuip.parse(huge)
+    assert "overflows" in e.value.log
