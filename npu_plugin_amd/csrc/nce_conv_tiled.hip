@@ -58,8 +58,15 @@ constexpr int vmcnt_imm(int n) {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
+// Waves per SIMD the register budget must allow (vector + accumulation registers share 512 per lane and SIMD): two
+// workgroups of four waves, or one of eight, per CU at the least - a lone wave per SIMD leaves every LDS and barrier
+// round trip of the step loop exposed.
+constexpr int tiled_min_waves(int nwaves) {
+    return nwaves >= 8 ? 2 : 2;
+}
+
 template <int WM, int WN, int TM, int TN, int NS, bool FZ>
-__global__ __launch_bounds__(64 * WM * WN) void conv_tiled_kernel(TiledArgs w) {
+__global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_tiled_kernel(TiledArgs w) {
     constexpr int NW = WM * WN;
     constexpr int NT = 64 * NW;
     constexpr int BM = 16 * TM * WM;

@@ -89,3 +89,17 @@ def test_scaled_cfg3_maxpool_batch512(executor):
 
 def test_scaled_cfg4_batch512(executor):
     check(K.cfg4(n=512), executor)
+
+
+def test_automatic_choice_of_the_tiled_kernel(executor, tuned):
+    """Sizes at which the dispatcher itself picks the LDS-tiled kernel (long reduction, 256 or more output channels, two
+    to four 128 x 128 workgroups per CU): same bytes as the oracle, and the same bytes as the weights-resident kernels
+    (NCE_HIP_CONV_TILED=0) give."""
+    import torch
+    for case in (K.conv_case(K.SEED + 31, 8, 56, 56, 128, 256, name="conv3x3_8x56x56x128_256"),
+                 K.conv_case(K.SEED + 32, 16, 28, 28, 1024, 512, k=(1, 1), pads=(0, 0, 0, 0), name="conv1x1_16x28x28x1024_512",
+                             ppe=dict(mode=3, clamp_low=128, clamp_high=255))):
+        want = K.run_oracle(case)
+        got = K.run_hip(case, executor)
+        assert np.array_equal(got, want), case.name
+        assert np.array_equal(K.run_hip(case, tuned(NCE_HIP_CONV_TILED=0)), want), case.name + " (tiled kernel off)"
