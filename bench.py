@@ -306,7 +306,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200, help="timed steps")
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg5")
+    ap.add_argument("--workload", default="cfg5", help="cfg1..cfg5, cfg3_chain, a large-batch variant, or conv:N,H,W,IC,OC,K,STRIDE,PAD")
     ap.add_argument("--no-others", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-scaled", action="store_true", help="skip the large-batch variants of the workloads")
@@ -324,6 +324,11 @@ def main():
     workloads = make_workloads()
     if args.workload in make_scaled_workloads():  # a large-batch variant as the main workload (profiling)
         workloads = dict(workloads, **{args.workload: make_scaled_workloads()[args.workload]})
+    if args.workload.startswith("conv:"):  # one convolution layer by shape (profiling): conv:N,H,W,IC,OC,K,STRIDE,PAD
+        from npu_plugin_amd import workloads as W
+        n, h, w_, ic, oc, k, st, pad = [int(x) for x in args.workload[5:].split(",")]
+        workloads = dict(workloads, **{args.workload: (lambda: W.conv_case(W.SEED + 21, n, h, w_, ic, oc, k=(k, k), s=(st, st),
+                                                                              pads=(pad, pad, pad, pad)), "mfma")})
     if args.workload not in workloads and args.workload not in ("cfg5", "cfg3_chain"):
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(workloads) + ['cfg3_chain', 'cfg5']}")
     ex = nce.Executor(device_id=0, log_level=1)
