@@ -122,6 +122,36 @@ def test_avgpool_with_weight_table(executor):
     check(K.pool_case(6, False, 2, 14, 14, 64, with_table=True), executor)
 
 
+@pytest.mark.parametrize("out_signed,lo,hi", [(True, -300, 300), (True, -128, 127), (True, -100, 90), (False, -40, 300), (False, 7, 200)])
+def test_window_clamp_bounds(executor, out_signed, lo, hi):
+    """Depthwise and average pool with clamp bounds inside and outside the storage range, signed and unsigned outputs
+    (the kernels choose between a truncating and a flooring conversion from the lower bound)."""
+    ppe = dict(mode=nce.PPE_NOOP, clamp_low=lo, clamp_high=hi)
+    check(K.dw_case(71, 2, 40, 36, 96, out_signed=out_signed, out_zp=-9 if out_signed else 131, ppe=ppe), executor)
+    m, sh = K.approx(15, 1.0 / 9)
+    check(K.pool_case(72, False, 2, 40, 36, 96, in_signed=out_signed, in_zp=-4 if out_signed else 120, out_zp=-9 if out_signed else 131,
+                      ppe=dict(ppe, quant_mult=m, quant_shift=sh)), executor)
+
+
+def test_window_strided_input_view(executor):
+    """Depthwise over an input that is a sub-view of a larger tensor (W, H and N strides larger than the compact ones):
+    interior wavefronts address their taps as 32-bit offsets into the view."""
+    import torch
+    case = K.dw_case(73, 2, 40, 36, 64, s=(1, 1))
+    want = K.run_oracle(case)
+    big_in = torch.zeros((2, 44, 40, 96), dtype=torch.uint8, device="cuda")
+    view_in = big_in[:, 3:43, 2:38, 16:80]
+    view_in.copy_(torch.from_numpy(case.input).cuda())
+    out = torch.zeros(case.out_shape, dtype=torch.uint8, device="cuda")
+    w = torch.from_numpy(case.weights).cuda()
+    t = torch.from_numpy(case.table).cuda()
+    task = K.build_task(case, view_in, w, t, out)
+    stream = torch.cuda.current_stream().cuda_stream
+    executor.enqueue(task, stream)
+    executor.synchronize(stream)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
 def test_maxpool_clamped(executor):
     check(K.pool_case(8, True, 1, 14, 14, 32, ppe=dict(mode=nce.PPE_NOOP, clamp_low=30, clamp_high=200)), executor)
 
