@@ -16,6 +16,7 @@
 #include "nce_conv_common.h"
 
 #include <algorithm>
+#include <numeric>
 #include <cstdlib>
 
 namespace nce {
@@ -269,7 +270,12 @@ void tile_bounds(const ConvArgs& a, int bm, int* rows_max, int* nslots_max) {
     int rmax = 0, smax = 0;
     const int64_t ntiles = ((int64_t)a.M + bm - 1) / bm;
     const int rows_full = (a.bh - 1) * a.SY + a.KY;
-    for (int64_t t = 0; t < ntiles; ++t) {
+    // A tile's extent depends only on where in an image it starts, and the start positions repeat after
+    // bw * bh / gcd(bm, bw * bh) tiles (a clipped last tile touches no more than the full tile of its position): the walk
+    // is bounded by the image, not by the batch.
+    const int64_t img = (int64_t)a.bw * a.bh;
+    const int64_t walk = std::min(ntiles, img / std::gcd<int64_t>(bm, img) + 1);
+    for (int64_t t = 0; t < walk; ++t) {
         const int64_t m0 = t * bm, m_end = std::min<int64_t>(m0 + bm, (int64_t)a.M);
         const int64_t rr_first = m0 / a.bw, rr_last = (m_end - 1) / a.bw;
         const int64_t n_first = rr_first / a.bh, n_last = rr_last / a.bh;

@@ -17,11 +17,7 @@
 //   * bytes are taken as unsigned (i8 storage is re-biased by x ^ 0x80) and out-of-image taps are
 //     filled with the zero point, so they contribute 0; the constant  -zp * sum(w)  is folded into
 //     the per-channel bias. (Max pool keeps the clamped in-window pixel instead: the maximum is the same.)
-//   * the requantize runs in FP64 (see nce_ppe_device.h); shifts above 44 take the integer path. Per-channel constants
-//     and depthwise weight pairs sit in LDS as [channel within group][group], so that the lanes of a wavefront
-//     (neighbouring groups of the same pixels) read neighbouring 16-byte entries.
-//   * wavefronts whose windows all lie inside the image (most) fetch their taps with buffer loads: one 32-bit offset
-//     per lane and item, the tap's offset in a scalar register.
+//   * the requantize runs in FP64 (see nce_ppe_device.h); shifts above 52 take the integer path.
 //   * MAXPOOL compares two channels per instruction (even / odd bytes as packed u16).
 #include "nce_conv_common.h"
 
@@ -36,7 +32,6 @@ constexpr int NT = 256;
 
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float ubyte_f32(uint32_t w, int i) {
     // the compiler turns this into v_cvt_f32_ubyte{i}
@@ -52,19 +47,13 @@ __device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// FP64 requantize of 16 channel sums (FP32 or int32, both exact) with per-channel constants, packed into 4 dwords.
-// TRUNC (folded mode with a lower clamp bound >= 0): the conversion to int32 truncates instead of flooring - the same
-// for values >= 0, and every value below 0 (floor's -1 for a value in (-1, 0) included) clamps to the bound either way.
-// mb: the lane's channel group in the table of (scale M, constant B) pairs, laid out [channel within group][group], so
-// that the lanes of a wavefront - neighbouring channel groups of the same pixels - read neighbouring 16-byte entries
-// (one conflict-free ds_read_b128 per channel; with [group][channel] the groups sit 128 bytes apart and share banks).
-template <int PMODE, bool TRUNC, typename Acc>
-__device__ __forceinline__ void requant16(const Acc (&acc)[16], const double2* mb, const PpeF64& pu, uint32_t (&wo)[4]) {
+// FP64 requantize of 16 channel sums with per-channel constants, packed into 4 dwords.
+template <int PMODE>
+__device__ __forceinline__ void requant16(const float (&acc)[16], const double* M, const double* B, const PpeF64& pu,
+                                          uint32_t (&wo)[4]) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const double2 c = mb[i * SLAB_GROUPS];
-        const double v = __builtin_fma((double)acc[i], c.x, c.y);
-        const int32_t y = TRUNC ? clamp_med3((int32_t)v, pu.lo_zp, pu.hi_zp) : ppe_finish_mode<PMODE>(v, pu);
+        const int32_t y = ppe_finish_mode<PMODE>(__builtin_fma((double)acc[i], M[i], B[i]), pu);
         const uint32_t b = (uint32_t)y & 0xFFu;
         wo[i >> 2] = (i & 3) == 0 ? b : (wo[i >> 2] | (b << (8 * (i & 3))));
     }
@@ -79,7 +68,6 @@ struct WinArgs {
     uint32_t a_xor;   // 0x80808080 for i8 activations
     uint32_t fill;    // word of re-biased zero-point bytes for out-of-image taps
     int32_t zpu;      // zero point of the re-biased (unsigned) activation bytes
-    uint32_t in_span; // bytes the input tensor spans if that is below 4 GiB (byte offsets into it fit 32 unsigned bits), else 0
     // I32 kernels (item count and tensor strides below 2^31): divisors of the item decomposition
     int32_t nslab_full;            // channel groups of every slab but the last
     FastDiv div_full, div_last;    // by the channel groups of a full slab / of the last slab
@@ -97,7 +85,7 @@ template <int MODE, int KK, bool I32>
 __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
     // MODE_DW: [tap][SLAB_CH] floats of (w - zp_w); then per-channel FP64 scale constants
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ double2 sMB[16 * SLAB_GROUPS];  // (M, B) of channel c of the slab at [c % 16][c / 16]
+    __shared__ double sM[SLAB_CH], sB[SLAB_CH];
     __shared__ int32_t sMult[SLAB_CH], sShift[SLAB_CH], sBias[SLAB_CH], sCorr[SLAB_CH];
 
     const TaskDev& t = a.t;
@@ -137,8 +125,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                         if (tap < KK * KK) wv[h] = (t.w_is_signed ? (int32_t)(int8_t)row[tap] : (int32_t)row[tap]) - t.w_zp;
                     }
                     wsum += wv[0] + wv[1];
-                    // [pair][dword of the group][group][channel of the dword]: the lanes' 16-byte reads are neighbours
-                    s_w2[((j * 4 + ((ch >> 2) & 3)) * SLAB_GROUPS + (ch >> 4)) * 4 + (ch & 3)] = ((uint32_t)wv[0] & 0xFFFFu) | ((uint32_t)wv[1] << 16);
+                    s_w2[j * SLAB_CH + ch] = ((uint32_t)wv[0] & 0xFFFFu) | ((uint32_t)wv[1] << 16);
                 }
             } else
             for (int tap = 0; tap < ntaps; ++tap) {
@@ -160,17 +147,8 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         use_int = (votes & 1) != 0;
         may_sat = (votes & 2) != 0;
     }
-    PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
+    const PpeF64 pu = ppe_f64_setup(t.ppe, may_sat);
     const int pmode = ppe_mode_of(pu, use_int);
-    // Folded mode: signed outputs are computed 128 higher and flipped back as bytes, so that the lower clamp bound is
-    // not negative and the conversion may truncate (requant16). Bounds outside the storage range keep the floor.
-    const int32_t flip = (MODE != MODE_MAX && pmode == PPE_MODE_FOLDED && t.out.is_signed) ? 128 : 0;
-    const bool trunc_ok = MODE != MODE_MAX && pmode == PPE_MODE_FOLDED && pu.lo_zp + flip >= 0 && pu.lo_zp <= pu.hi_zp;
-    if (trunc_ok) {
-        pu.lo_zp += flip;
-        pu.hi_zp += flip;
-    }
-    const uint32_t out_xor = trunc_ok && flip ? 0x80808080u : 0u;
     if (has_ch) {
         // out-of-image taps were filled with the zero point: remove zpu * sum(w) exactly
         const int32_t corr = -a.zpu * wsum;
@@ -179,12 +157,11 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         sBias[ch] = bias;
         sCorr[ch] = corr;  // |corr| < 2^23
         const double M = ppe_scale_M(mult, shift);
-        sMB[(ch & 15) * SLAB_GROUPS + (ch >> 4)] = make_double2(M, ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu) + (trunc_ok ? (double)flip : 0.0));
+        sM[ch] = M;
+        sB[ch] = ppe_mode_B(__builtin_fma((double)corr, M, ppe_scale_B(bias, M, shift, t.ppe.round_mode)), pmode, pu);
     }
     if constexpr (MODE != MODE_MAX) __syncthreads();
 
-    // (raw buffer over the input tensor: 32-bit offsets, no swizzle, 32-bit data format)
-    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(t.in.data), 0, (int32_t)a.in_span, 0x00020000);
     const int64_t nitems = a.npix * nslab;
     const int64_t first = (int64_t)xcd_tile(blockIdx.x, a.nblocks) * NT * a.items_per_thread;
     for (int it = 0; it < a.items_per_thread; ++it) {
@@ -301,36 +278,21 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
         };
         if constexpr (KK > 0) {
             uint4 v[KK * KK];
-            // Most wavefronts hold no tap outside the image. Their loads are buffer loads: the tensor as a buffer resource,
-            // one 32-bit offset per lane computed once per item, and the tap's offset in a scalar register - no clamping
-            // and no 64-bit address arithmetic per tap.
+#pragma unroll
+            for (int ky = 0; ky < KK; ++ky)
+#pragma unroll
+                for (int kx = 0; kx < KK; ++kx) {
+                    const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
+                    v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
+                }
+            // Out-of-image taps take the zero point. Most wavefronts hold no such tap: the replacement runs only where
+            // one does (uniform branch).
             const bool inside = iy0 >= 0 && ix0 >= 0 && iy0 + KK <= t.in.h && ix0 + KK <= t.in.w;
-            const bool all_inside = __all(inside);
-            if (I32 && a.in_span != 0 && all_inside) {
-                const uint32_t off0 = (uint32_t)n * (uint32_t)t.in.sn + (uint32_t)iy0 * (uint32_t)t.in.sh + (uint32_t)ix0 * (uint32_t)t.in.sw + (uint32_t)oc;
-#pragma unroll
-                for (int ky = 0; ky < KK; ++ky)
-#pragma unroll
-                    for (int kx = 0; kx < KK; ++kx) {
-                        const u32x4 r = __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off0, (int32_t)(ky * (uint32_t)t.in.sh + kx * (uint32_t)t.in.sw), 0);
-                        v[ky * KK + kx] = make_uint4(r.x, r.y, r.z, r.w);
-                    }
-            } else {
-#pragma unroll
-                for (int ky = 0; ky < KK; ++ky)
-#pragma unroll
-                    for (int kx = 0; kx < KK; ++kx) {
-                        const int32_t iy = min(max(iy0 + ky, 0), t.in.h - 1), ix = min(max(ix0 + kx, 0), t.in.w - 1);
-                        v[ky * KK + kx] = *reinterpret_cast<const uint4*>(src + mul(iy, t.in.sh) + mul(ix, t.in.sw));
-                    }
-            }
             if (a.a_xor != 0) {  // uniform: i8 storage is re-biased to unsigned bytes
-                asm volatile("" ::: "memory");  // (keeps this a branch: as a select the XORs run for u8 storage too)
 #pragma unroll
                 for (int i = 0; i < KK * KK; ++i) v[i] = make_uint4(v[i].x ^ a.a_xor, v[i].y ^ a.a_xor, v[i].z ^ a.a_xor, v[i].w ^ a.a_xor);
             }
-            // Out-of-image taps take the zero point: the replacement runs only in wavefronts that hold one.
-            if (!all_inside) {
+            if (!__all(inside)) {
                 const uint32_t fr = a.fill;
 #pragma unroll
                 for (int ky = 0; ky < KK; ++ky)
@@ -348,7 +310,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 int32_t acci[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acci[i] = 0;
-                const uint32_t* wp2 = reinterpret_cast<const uint32_t*>(smem) + (cg << 2);
+                const uint32_t* wp2 = reinterpret_cast<const uint32_t*>(smem) + (cg << 4);
 #pragma unroll
                 for (int j = 0; j < (KK * KK + 1) / 2; ++j) {
                     const uint4 ra = fixed((2 * j) / KK, (2 * j) % KK);
@@ -356,7 +318,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                     const uint32_t wa[4] = {ra.x, ra.y, ra.z, ra.w}, wb[4] = {rb.x, rb.y, rb.z, rb.w};
 #pragma unroll
                     for (int d = 0; d < 4; ++d) {
-                        const uint4 w4 = *reinterpret_cast<const uint4*>(wp2 + (j * 4 + d) * (SLAB_GROUPS * 4));
+                        const uint4 w4 = *reinterpret_cast<const uint4*>(wp2 + j * SLAB_CH + 4 * d);
                         const uint32_t wv[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -365,13 +327,6 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                                                                      acci[4 * d + i], false);
                         }
                     }
-                }
-                if (pmode == PPE_MODE_FOLDED) {  // (uniform) the usual case: requantise straight from the integer sums
-                    uint32_t wq[4];
-                    if (trunc_ok) requant16<PPE_MODE_FOLDED, true>(acci, sMB + cg, pu, wq);
-                    else requant16<PPE_MODE_FOLDED, false>(acci, sMB + cg, pu, wq);
-                    store_channels16(dst, t.out.sc, wq[0] ^ out_xor, wq[1] ^ out_xor, wq[2] ^ out_xor, wq[3] ^ out_xor);
-                    continue;
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[i] = (float)acci[i];  // exact: below 2^24
@@ -402,9 +357,8 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
 
         uint32_t wo[4];
         const int chl = cg << 4;
-        if (pmode == PPE_MODE_FOLDED && trunc_ok) requant16<PPE_MODE_FOLDED, true>(acc, sMB + cg, pu, wo);
-        else if (pmode == PPE_MODE_FOLDED) requant16<PPE_MODE_FOLDED, false>(acc, sMB + cg, pu, wo);
-        else if (pmode == PPE_MODE_SLOPE) requant16<PPE_MODE_SLOPE, false>(acc, sMB + cg, pu, wo);
+        if (pmode == PPE_MODE_FOLDED) requant16<PPE_MODE_FOLDED>(acc, sM + chl, sB + chl, pu, wo);
+        else if (pmode == PPE_MODE_SLOPE) requant16<PPE_MODE_SLOPE>(acc, sM + chl, sB + chl, pu, wo);
         else {
             wo[0] = wo[1] = wo[2] = wo[3] = 0;
 #pragma unroll
@@ -414,7 +368,7 @@ __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
                 wo[i >> 2] |= ((uint32_t)y & 0xFFu) << (8 * (i & 3));
             }
         }
-        store_channels16(dst, t.out.sc, wo[0] ^ out_xor, wo[1] ^ out_xor, wo[2] ^ out_xor, wo[3] ^ out_xor);
+        store_channels16(dst, t.out.sc, wo[0], wo[1], wo[2], wo[3]);
     }
 }
 
@@ -453,8 +407,6 @@ hipError_t launch_window_kk(const TaskDev& t, const Box& box, hipStream_t s) {
     a.div_bh = make_fastdiv((uint32_t)box.bh);
     bool i32 = blocks * NT * a.items_per_thread < 0x7fffffffLL;
     for (const int64_t st : {t.in.sn, t.in.sh, t.in.sw, t.out.sn, t.out.sh, t.out.sw}) i32 = i32 && st >= 0 && st <= 0x7fffffffLL;
-    const bool ordered = t.in.sn >= (int64_t)t.in.h * t.in.sh && t.in.sh >= (int64_t)t.in.w * t.in.sw && t.in.sw >= t.in.c;
-    a.in_span = ordered && (int64_t)t.in.n * t.in.sn <= 0xffffffffLL ? (uint32_t)((int64_t)t.in.n * t.in.sn) : 0u;
     if (i32) return launch_window_i32<MODE, KK, true>(a, blocks, nslabs, lds, s);
     return launch_window_i32<MODE, KK, false>(a, blocks, nslabs, lds, s);
 }
