@@ -65,7 +65,7 @@ constexpr int tiled_min_waves(int nwaves) {
     return nwaves >= 8 ? 2 : 2;
 }
 
-template <int WM, int WN, int TM, int TN, int NS, bool FZ>
+template <int WM, int WN, int TM, int TN, int NS, int KC, bool FZ>
 __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_tiled_kernel(TiledArgs w) {
     constexpr int NW = WM * WN;
     constexpr int NT = 64 * NW;
@@ -75,11 +75,12 @@ __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_t
     constexpr int ABLK = BN / 16;            // 1 KiB blocks of the weight tile
     constexpr int NA = ABLK / NW;            // blocks of the weight tile one wave fetches per step
     constexpr int NB = (BM / 16) / NW;       // blocks of the activation tile
-    constexpr int STAGE = (BM + BN) * 64;    // bytes of one LDS stage
+    constexpr int CHUNK = (BM + BN) * 64;    // bytes of one 64-byte slice of the reduction: weight rows, then activation rows
+    constexpr int STAGE = CHUNK * KC;        // bytes of one LDS stage: KC slices (a step covers 64 * KC bytes of the reduction)
     static_assert(TN == 2 || TN == 4, "channel fragments per wave");
     static_assert(ABLK % NW == 0 && (BM / 16) % NW == 0, "blocks divide among the waves");
     static_assert(!FZ || TN == 4, "fused add: a lane holds 16 channels");
-    static_assert(NS >= 2 && (NS - 2) * (NA + NB) < 64, "ring depth against the 6-bit load counter");
+    static_assert(NS >= 2 && (NS - 2) * (NA + NB) * KC < 64, "ring depth against the 6-bit load counter");
     const ConvArgs& a = w.a;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sT[];  // [stage][weights BN rows | activations BM rows] x 64 bytes
@@ -141,19 +142,23 @@ __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_t
     int64_t it_off = 0, tap_off = 0, w_off = 0;
     // Request one step's operands into ring slot `slot` (uniform).
     auto request = [&](int slot) {
-        uint8_t* const st = sT + slot * STAGE + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < NA; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + w_off), (lptr_t)(st + NW * i * 1024), 16, 0, 0);
+        for (int c = 0; c < KC; ++c) {
+            uint8_t* const st = sT + slot * STAGE + c * CHUNK + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            const uint8_t* src = bsrc[i] + it_off;
-            if (!w.inside) src = ((rows[i] >> it_ky) & (cols[i] >> it_kx) & 1u) ? src : fillp;
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + (ABLK + NW * i) * 1024), 16, 0, 0);
+            for (int i = 0; i < NA; ++i)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + w_off + 64 * c), (lptr_t)(st + NW * i * 1024), 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const uint8_t* src = bsrc[i] + it_off + 64 * c;
+                if (!w.inside) src = ((rows[i] >> it_ky) & (cols[i] >> it_kx) & 1u) ? src : fillp;
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + (ABLK + NW * i) * 1024), 16, 0, 0);
+            }
         }
-        w_off += 64;
-        it_off += 64;
-        if (++it_c64 == w.nc64) {
+        w_off += 64 * KC;
+        it_off += 64 * KC;
+        it_c64 += KC;
+        if (it_c64 == w.nc64) {
             it_c64 = 0;
             tap_off += a.in_sw;
             if (++it_kx == a.KX) {
@@ -203,31 +208,37 @@ __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_t
         for (int s = 0; s < S; ++s) {
             // The requests of step s are this wave's oldest; younger ones (at most NS - 2 steps) may stay in flight.
             // Near the end fewer are younger, so there everything is waited for.
-            if (s + NS - 1 <= S) __builtin_amdgcn_s_waitcnt(vmcnt_imm((NS - 2) * (NA + NB)));
+            if (s + NS - 1 <= S) __builtin_amdgcn_s_waitcnt(vmcnt_imm((NS - 2) * (NA + NB) * KC));
             else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
             // Every wave's pieces of step s are in LDS, and every wave has left step s - 1's slot. (The bare barrier:
             // __syncthreads() would first wait for ALL outstanding loads, which empties the ring at every step.)
             __builtin_amdgcn_s_barrier();
             if (s + NS - 1 < S) request(slot == 0 ? NS - 1 : slot - 1);
             const uint8_t* const st = sT + slot * STAGE;
-            v4i fa[TN], fb[TM];
+            v4i fa[KC][TN], fb[KC][TM];
 #pragma unroll
-            for (int f = 0; f < TN; ++f) fa[f] = *reinterpret_cast<const v4i*>(st + a_rd + f * 1024);
+            for (int c = 0; c < KC; ++c) {
 #pragma unroll
-            for (int x = 0; x < TM; ++x) fb[x] = *reinterpret_cast<const v4i*>(st + b_rd + x * 1024);
-            if (wxor != 0) {  // uniform
+                for (int f = 0; f < TN; ++f) fa[c][f] = *reinterpret_cast<const v4i*>(st + c * CHUNK + a_rd + f * 1024);
 #pragma unroll
-                for (int f = 0; f < TN; ++f) fa[f] ^= wxor;
+                for (int x = 0; x < TM; ++x) fb[c][x] = *reinterpret_cast<const v4i*>(st + c * CHUNK + b_rd + x * 1024);
             }
 #pragma unroll
-            for (int x = 0; x < TM; ++x) fb[x] ^= axor;
+            for (int c = 0; c < KC; ++c) {
+                if (wxor != 0) {  // uniform
 #pragma unroll
-            for (int f = 0; f < TN; ++f)
+                    for (int f = 0; f < TN; ++f) fa[c][f] ^= wxor;
+                }
 #pragma unroll
-                for (int x = 0; x < TM; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], fb[x], acc[f][x], 0, 0, 0);
-            if constexpr (WS) {
+                for (int x = 0; x < TM; ++x) fb[c][x] ^= axor;
 #pragma unroll
-                for (int f = 0; f < TN; ++f) wsa[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], ones, wsa[f], 0, 0, 0);
+                for (int f = 0; f < TN; ++f)
+#pragma unroll
+                    for (int x = 0; x < TM; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[c][f], fb[c][x], acc[f][x], 0, 0, 0);
+                if constexpr (WS) {
+#pragma unroll
+                    for (int f = 0; f < TN; ++f) wsa[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[c][f], ones, wsa[f], 0, 0, 0);
+                }
             }
             slot = slot == NS - 1 ? 0 : slot + 1;
         }
@@ -334,12 +345,14 @@ __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_t
     else wres_epilogue<TN, TM, PPE_MODE_INT, FZ>(a, ew, bw, cw, acc, dws, q, nocw, dst, valid, pu, ep, &w.fz, other);
 }
 
-template <int WM, int WN, int TM, int TN, int NS>
+template <int WM, int WN, int TM, int TN, int NS, int KC = 1>
 hipError_t launch_shape(TiledArgs& w, bool fused, hipStream_t stream) {
     constexpr int BM = 16 * TM * WM;
     constexpr int BN = 16 * TN * WN;
-    constexpr size_t lds = (size_t)NS * (BM + BN) * 64;
+    constexpr size_t lds = (size_t)NS * (BM + BN) * 64 * KC;
     const ConvArgs& a = w.a;
+    if (w.nc64 % KC != 0) return hipErrorNotSupported;
+    w.nsteps = a.KY * a.KX * (w.nc64 / KC);
     w.ntm = (uint32_t)(((int64_t)a.M + BM - 1) / BM);
     w.ntn = (uint32_t)((a.bc + BN - 1) / BN);
     const uint64_t total = (uint64_t)w.ntm * w.ntn;
@@ -347,14 +360,14 @@ hipError_t launch_shape(TiledArgs& w, bool fused, hipStream_t stream) {
     const dim3 grid(xcd_grid((uint32_t)total)), block(64 * WM * WN);
     if (fused) {
         if constexpr (TN == 4) {
-            auto kernel = &conv_tiled_kernel<WM, WN, TM, TN, NS, true>;
+            auto kernel = &conv_tiled_kernel<WM, WN, TM, TN, NS, KC, true>;
             static LdsGrant grant;
             if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
             return emit(kernel, grid, block, lds, stream, w);
         }
         return hipErrorNotSupported;
     }
-    auto kernel = &conv_tiled_kernel<WM, WN, TM, TN, NS, false>;
+    auto kernel = &conv_tiled_kernel<WM, WN, TM, TN, NS, KC, false>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     return emit(kernel, grid, block, lds, stream, w);
@@ -363,7 +376,8 @@ hipError_t launch_shape(TiledArgs& w, bool fused, hipStream_t stream) {
 }  // namespace
 
 // Shapes: 1 = 128 px x 128 ch (4 waves), 2 = 64 px x 128 ch (4 waves), 3 = 256 px x 128 ch (8 waves),
-// 4 = 128 px x 64 ch (4 waves). shape 0 = automatic.
+// 4 = 128 px x 64 ch (4 waves), 5 = shape 1 with steps of 128 bytes of the reduction (input channels a multiple of 128).
+// shape 0 = automatic.
 hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, const FuseAdd* fuse) {
     if (a.IC % 64 != 0 || a.dw != 0 || a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     if (a.M > 0x7fffffff - 1024) return hipErrorNotSupported;
@@ -382,7 +396,7 @@ hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, c
     if (shape == 0) {
         // The largest tile that still gives every CU about two workgroups.
         const auto groups = [&](int bm, int bn) { return (((int64_t)a.M + bm - 1) / bm) * ((a.bc + bn - 1) / bn); };
-        shape = groups(128, 128) >= 512 ? 1 : 2;
+        shape = groups(128, 128) >= 512 ? (a.IC % 128 == 0 ? 5 : 1) : 2;
     }
     const bool fz = fuse != nullptr;
     switch (shape) {
@@ -390,6 +404,7 @@ hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, c
     case 2: return launch_shape<2, 2, 2, 4, 4>(w, fz, stream);
     case 3: return launch_shape<4, 2, 4, 4, 3>(w, fz, stream);
     case 4: return launch_shape<2, 2, 4, 2, 4>(w, fz, stream);
+    case 5: return launch_shape<2, 2, 4, 4, 2, 2>(w, fz, stream);
     default: return hipErrorNotSupported;
     }
 }
