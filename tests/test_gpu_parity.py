@@ -758,3 +758,46 @@ def test_conv_fused_add_equals_two_launches(tuned):
                               (conv_kw, dict(add_kw, shift=40))):
         g1, g2, y1, y2 = _conv_then_add(tuned, conv_kw2, add_kw2, False, False, "4,2,8,0")
         assert np.array_equal(g1, y1) and np.array_equal(g2, y2)
+
+
+# ---- the limits the reference's verifier allows (kernel 1..11, stride 1..8, pad <= K/2, channels in 16s; VPUIP
+# nce_invariant.cpp:1056-1108) and degenerate images --------------------------------------------------------------------
+
+LIMIT_CONVS = [
+    dict(n=1, h=11, w=11, ic=16, oc=16, k=(11, 11), s=(1, 1), pads=(5, 5, 5, 5)),      # largest kernel, largest padding
+    dict(n=2, h=33, w=41, ic=32, oc=32, k=(11, 11), s=(8, 8), pads=(5, 5, 5, 5)),      # largest kernel and stride
+    dict(n=1, h=24, w=17, ic=64, oc=48, k=(3, 3), s=(8, 1), pads=(1, 1, 1, 1)),        # strides 8 x 1
+    dict(n=1, h=17, w=24, ic=64, oc=48, k=(3, 3), s=(1, 8), pads=(1, 1, 1, 1)),        # strides 1 x 8
+    dict(n=1, h=1, w=1, ic=16, oc=16, k=(1, 1), s=(1, 1), pads=(0, 0, 0, 0)),          # one pixel, 16 channels
+    dict(n=3, h=1, w=1, ic=2048, oc=1008, k=(1, 1), s=(1, 1), pads=(0, 0, 0, 0)),      # the classifier head: 1 x 1 images
+    dict(n=1, h=3, w=3, ic=64, oc=64, k=(3, 3), s=(1, 1), pads=(0, 0, 0, 0)),          # one output pixel from a 3 x 3 image
+    dict(n=2, h=1, w=37, ic=64, oc=32, k=(1, 3), s=(1, 1), pads=(1, 1, 0, 0)),         # one image row
+    dict(n=2, h=37, w=1, ic=64, oc=32, k=(3, 1), s=(1, 1), pads=(0, 0, 1, 1)),         # one image column
+    dict(n=1, h=2, w=2, ic=8192, oc=32, k=(1, 1), s=(1, 1), pads=(0, 0, 0, 0)),        # 8192 input channels
+    dict(n=1, h=2, w=2, ic=64, oc=8192, k=(1, 1), s=(1, 1), pads=(0, 0, 0, 0)),        # 8192 output channels
+    dict(n=1, h=1024, w=1024, ic=16, oc=16, k=(3, 3), s=(1, 1), pads=(1, 1, 1, 1)),    # a megapixel image
+    dict(n=1, h=5, w=5, ic=16, oc=16, k=(5, 5), s=(1, 1), pads=(2, 0, 0, 2)),          # padding on two sides only
+]
+
+
+@pytest.mark.parametrize("c", LIMIT_CONVS, ids=lambda c: f"{c['n']}x{c['h']}x{c['w']}x{c['ic']}_{c['oc']}_k{c['k'][0]}x{c['k'][1]}s{c['s'][0]}x{c['s'][1]}")
+def test_conv_limits(executor, c):
+    check(K.conv_case(900 + c["ic"] % 97 + c["h"], c["n"], c["h"], c["w"], c["ic"], c["oc"], k=c["k"], s=c["s"], pads=c["pads"]), executor)
+
+
+@pytest.mark.parametrize("kind", ["dw", "max", "avg"])
+@pytest.mark.parametrize("h,w,c,k,s,pads", [(11, 11, 16, (11, 11), (1, 1), (5, 5, 5, 5)), (40, 33, 32, (11, 11), (8, 8), (5, 5, 5, 5)),
+                                            (1, 1, 4096, (1, 1), (1, 1), (0, 0, 0, 0)), (1, 29, 48, (1, 3), (1, 2), (1, 1, 0, 0)),
+                                            (29, 1, 48, (3, 1), (2, 1), (0, 0, 1, 1)), (700, 700, 16, (3, 3), (2, 2), (1, 1, 1, 1))])
+def test_window_limits(executor, kind, h, w, c, k, s, pads):
+    if kind == "dw":
+        check(K.dw_case(950 + h, 1, h, w, c, k=k, s=s, pads=pads), executor)
+    else:
+        m, sh = K.approx(15, 1.0 / (k[0] * k[1]))
+        ppe = None if kind == "max" else dict(mode=nce.PPE_NOOP, clamp_low=0, clamp_high=255, quant_mult=m, quant_shift=sh)
+        check(K.pool_case(960 + h, kind == "max", 1, h, w, c, k=k, s=s, pads=pads, ppe=ppe), executor)
+
+
+@pytest.mark.parametrize("n,h,w,c", [(1, 1, 1, 16), (1, 1, 1, 8192), (1, 1024, 1024, 16), (5, 3, 7, 48)])
+def test_eltwise_limits(executor, n, h, w, c):
+    check(K.eltwise_case(970 + c % 89, n, h, w, c), executor)
