@@ -5,18 +5,27 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <new>
 #include <string>
 #include <vector>
 
 #include "nce_common.h"
+#include "nce_conv_pk.h"
 #include "nce_log.h"
 
 struct nce_executor_s {
     int device = 0;
     nce_log_s* log = nullptr;
     nce::Options opt;  // tuning knobs, read from the environment once at creation
+    // Persistent segments: a pinned host word their kernels raise when a bounded wait ran out (checked after a
+    // synchronise; persistent launches are then switched off for this executor).
+    uint32_t* pk_host_error = nullptr;
+    std::atomic<bool> pk_off{false};
+    ~nce_executor_s() {
+        if (pk_host_error != nullptr) (void)hipHostFree(pk_host_error);
+    }
 };
 
 thread_local nce::LaunchContext nce::tls_launch;
@@ -58,6 +67,8 @@ nce::Options read_options() {
     if (const char* e = getenv("NCE_HIP_CONV_TILE")) o.halo_tile = atoi(e);
     if (const char* e = getenv("NCE_HIP_CONV_TILED")) o.tiled = atoi(e);
     o.no_fuse = getenv("NCE_HIP_NO_FUSE") != nullptr;
+    if (const char* e = getenv("NCE_HIP_PERSISTENT")) o.persistent = atoi(e);
+    if (const char* e = getenv("NCE_HIP_PERSISTENT_WAIT_US")) o.persistent_wait_us = std::max(0, atoi(e));
     return o;
 }
 
@@ -447,13 +458,97 @@ struct nce_task_list_s {
     std::mutex mu;
     std::vector<Plan> plans;
     std::vector<nce::RecordedLaunch> launches;
+    std::vector<void*> device_mem;  // tables and counters of persistent segments
     bool prepared = false;
+    bool has_segments = false;
+    void drop_prepared() {
+        for (void* p : device_mem) (void)hipFree(p);
+        device_mem.clear();
+        launches.clear();
+        prepared = false;
+        has_segments = false;
+    }
+    ~nce_task_list_s() { drop_prepared(); }
 };
 
 namespace {
 
-// Walk the plans the way they are to run (stream order), launching or - with a recorder set - recording.
-nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipStream_t stream) {
+// ---- persistent segments (nce_conv_pk.h) -----------------------------------------------------------------------------------
+// A tensor a layer touches, for the question whether a run of layers may share one persistent launch: every XCD works on
+// its own eighth of the batch and runs ahead of or behind the others, so two layers of a segment may touch the same memory
+// only if both cut it into the same eight shares (same base, batch and batch stride) - or if both only read it.
+struct PkTensor {
+    const uint8_t* lo;
+    const uint8_t* hi;
+    int64_t sn;
+    int32_t n;        // 0: not cut by batch (weights, tables)
+    bool written;
+};
+PkTensor pk_tensor(const nce::TensorDev& t, bool written) {
+    return {t.data, t.data + (int64_t)t.n * t.sn, t.sn, t.n, written};
+}
+bool pk_conflict(const PkTensor& x, const PkTensor& y) {
+    if (!(x.lo < y.hi && y.lo < x.hi)) return false;
+    if (!x.written && !y.written) return false;
+    return !(x.n != 0 && x.lo == y.lo && x.n == y.n && x.sn == y.sn);
+}
+
+// The per-XCD form of one recorded launch (a convolution, possibly with its fused residual add), if it has one.
+struct PkAlt {
+    bool ok = false;
+    nce::RecordedLaunch launch;          // recorded with an eighth of the batch for 32 CUs
+    int64_t d_in = 0, d_out = 0, d_other = 0, d_fzout = 0;
+    std::vector<PkTensor> tensors;
+};
+
+PkAlt pk_alternate(const Plan& p, const Plan* q) {
+    PkAlt alt;
+    const int32_t n = p.dev.out.n;
+    if (p.boxes.size() != 1 || n % 8 != 0 || p.dev.in.n != n) return alt;
+    if (q != nullptr && (q->boxes.size() != 1 || q->dev.in.n != n || q->dev.in2.n != n || q->dev.out.n != n)) return alt;
+    TaskDev pd = p.dev;
+    pd.in.n = pd.out.n = n / 8;
+    std::vector<nce::RecordedLaunch> rec;
+    const nce::LaunchContext saved = nce::tls_launch;
+    nce::tls_launch.record = &rec;
+    nce::tls_launch.per_xcd = true;
+    hipError_t e;
+    if (q != nullptr) {
+        TaskDev qd = q->dev;
+        qd.in.n = qd.in2.n = qd.out.n = n / 8;
+        e = nce::launch_conv_fused_add(pd, p.boxes[0], qd, q->boxes[0], nullptr);
+    } else {
+        e = nce::launch_conv(pd, p.boxes[0], nullptr);
+    }
+    nce::tls_launch = saved;
+    if (e != hipSuccess || rec.size() != 1 || !nce::wres_pk_has_variant(rec[0].tag)) return alt;
+    alt.launch = std::move(rec[0]);
+    alt.d_in = (int64_t)(n / 8) * p.dev.in.sn;
+    alt.d_out = (int64_t)(n / 8) * p.dev.out.sn;
+    alt.tensors.push_back(pk_tensor(p.dev.in, false));
+    alt.tensors.push_back(pk_tensor(p.dev.out, true));
+    alt.tensors.push_back({p.dev.weights, p.dev.weights + (int64_t)p.dev.out.c * p.dev.w_stride_oc, 0, 0, false});
+    const uint8_t* const tb = reinterpret_cast<const uint8_t*>(p.dev.table);
+    alt.tensors.push_back({tb, tb + (int64_t)p.dev.out.c * p.dev.table_stride * 4, 0, 0, false});
+    if (q != nullptr) {
+        const nce::TensorDev& other = q->dev.in.data == p.dev.out.data ? q->dev.in2 : q->dev.in;
+        alt.d_other = (int64_t)(n / 8) * other.sn;
+        alt.d_fzout = (int64_t)(n / 8) * q->dev.out.sn;
+        alt.tensors.push_back(pk_tensor(other, false));
+        alt.tensors.push_back(pk_tensor(q->dev.out, true));
+    }
+    alt.ok = true;
+    return alt;
+}
+
+// Walk the plans the way they are to run (stream order), launching or - with a recorder set - recording. alts (recording
+// only, optional) receives one entry per recorded launch: its per-XCD form where it has one.
+nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipStream_t stream, std::vector<PkAlt>* alts = nullptr) {
+    const auto note = [&](PkAlt&& alt) {
+        if (alts == nullptr) return;
+        while (alts->size() + 1 < nce::tls_launch.record->size()) alts->emplace_back();  // launches without an alternate
+        alts->push_back(std::move(alt));
+    };
     for (size_t i = 0; i < plans.size(); ++i) {
         const Plan& p = plans[i];
         // A convolution directly followed by the residual add that consumes its output runs as one launch where the
@@ -463,6 +558,7 @@ nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipSt
             if (q.task_type == NCE_TASK_ELTWISE && q.boxes.size() == 1) {
                 const hipError_t e = nce::launch_conv_fused_add(p.dev, p.boxes[0], q.dev, q.boxes[0], stream);
                 if (e == hipSuccess) {
+                    if (alts != nullptr) note(pk_alternate(p, &q));
                     ++i;
                     continue;
                 }
@@ -474,7 +570,77 @@ nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipSt
         }
         const nce_result_t r = launch_plan(ex, p, stream);
         if (r != NCE_RESULT_SUCCESS) return r;
+        if (alts != nullptr && p.task_type == NCE_TASK_CONV && p.boxes.size() == 1) note(pk_alternate(p, nullptr));
     }
+    if (alts != nullptr) alts->resize(nce::tls_launch.record->size());
+    return NCE_RESULT_SUCCESS;
+}
+
+// Replace every run of two or more consecutive launches that have a per-XCD form (and whose tensors allow it) by one
+// persistent launch. Allocates the segments' device tables and counters (kept in list->device_mem).
+nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts) {
+    nce_executor_s* const ex = list->ex;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, ex->device) != hipSuccess || prop.multiProcessorCount != nce::kPkWorkgroups) return NCE_RESULT_SUCCESS;
+    if (ex->pk_host_error == nullptr) {
+        if (hipHostMalloc(reinterpret_cast<void**>(&ex->pk_host_error), 64, hipHostMallocDefault) != hipSuccess) return NCE_RESULT_SUCCESS;
+        *ex->pk_host_error = 0;
+    }
+    std::vector<nce::RecordedLaunch> out;
+    size_t i = 0;
+    const size_t n = list->launches.size();
+    while (i < n) {
+        // the longest run from i whose tensors do not conflict
+        size_t j = i;
+        std::vector<PkTensor> seen;
+        while (j < n && alts[j].ok && j - i < (size_t)nce::kPkMaxLayers) {
+            bool clash = false;
+            for (const PkTensor& t : alts[j].tensors)
+                for (const PkTensor& u : seen) clash = clash || pk_conflict(t, u);
+            if (clash) break;
+            seen.insert(seen.end(), alts[j].tensors.begin(), alts[j].tensors.end());
+            ++j;
+        }
+        if (j - i < 2) {
+            out.push_back(std::move(list->launches[i]));
+            ++i;
+            continue;
+        }
+        std::vector<nce::PkLayerDesc> layers;
+        for (size_t k = i; k < j; ++k) layers.push_back({&alts[k].launch, alts[k].d_in, alts[k].d_out, alts[k].d_other, alts[k].d_fzout});
+        std::vector<uint8_t> table;
+        nce::RecordedLaunch seg;
+        const hipError_t e = nce::wres_pk_make(layers, &table, &seg);
+        void* d_table = nullptr;
+        void* d_ctl = nullptr;
+        if (e != hipSuccess || hipMalloc(&d_table, table.size()) != hipSuccess) {
+            for (size_t k = i; k < j; ++k) out.push_back(std::move(list->launches[k]));
+            i = j;
+            continue;
+        }
+        list->device_mem.push_back(d_table);
+        if (hipMalloc(&d_ctl, sizeof(nce::PkCtl)) != hipSuccess || hipMemcpy(d_table, table.data(), table.size(), hipMemcpyHostToDevice) != hipSuccess) {
+            for (size_t k = i; k < j; ++k) out.push_back(std::move(list->launches[k]));
+            i = j;
+            continue;
+        }
+        list->device_mem.push_back(d_ctl);
+        nce::PkArgs args;
+        args.layers = d_table;
+        args.ctl = static_cast<nce::PkCtl*>(d_ctl);
+        args.host_error = ex->pk_host_error;
+        args.nlayers = (int32_t)(j - i);
+        args.wait_us = (uint32_t)ex->opt.persistent_wait_us;
+        seg.arg.resize((sizeof(args) + 7) / 8);
+        memcpy(seg.arg.data(), &args, sizeof(args));
+        seg.clear = d_ctl;
+        seg.clear_bytes = (uint32_t)sizeof(nce::PkCtl);
+        out.push_back(std::move(seg));
+        list->has_segments = true;
+        ex->log->add(3, "task list: launches %zu..%zu run as one persistent launch", i, j - 1);
+        i = j;
+    }
+    list->launches = std::move(out);
     return NCE_RESULT_SUCCESS;
 }
 
@@ -577,8 +743,7 @@ nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_ta
         if (r != NCE_RESULT_SUCCESS) return r;
         std::lock_guard<std::mutex> lk(list->mu);
         list->plans.push_back(std::move(plan));
-        list->prepared = false;
-        list->launches.clear();
+        list->drop_prepared();
         return NCE_RESULT_SUCCESS;
     } catch (const std::bad_alloc&) {
         return NCE_RESULT_ERROR_OUT_OF_MEMORY;
@@ -594,14 +759,27 @@ nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     try {
         std::lock_guard<std::mutex> lk(list->mu);
+        if (list->prepared && list->has_segments && list->ex->pk_off.load()) list->drop_prepared();
         if (!list->prepared) {
             // Kernel choice, grids and argument blocks are worked out once, here; later calls only replay them.
-            list->launches.clear();
-            const ScopedLaunch ctx(&list->ex->opt, &list->launches);
-            const nce_result_t r = run_plans(list->ex, list->plans, nullptr);
-            if (r != NCE_RESULT_SUCCESS) {
-                list->launches.clear();
-                return r;
+            list->drop_prepared();
+            const bool persistent = list->ex->opt.persistent != 0 && !list->ex->pk_off.load();
+            std::vector<PkAlt> alts;
+            {
+                const ScopedLaunch ctx(&list->ex->opt, &list->launches);
+                const nce_result_t r = run_plans(list->ex, list->plans, nullptr, persistent ? &alts : nullptr);
+                if (r != NCE_RESULT_SUCCESS) {
+                    list->launches.clear();
+                    return r;
+                }
+            }
+            if (persistent) {
+                const ScopedLaunch ctx(&list->ex->opt, nullptr);
+                const nce_result_t r = build_segments(list, alts);
+                if (r != NCE_RESULT_SUCCESS) {
+                    list->drop_prepared();
+                    return r;
+                }
             }
             list->prepared = true;
         }
@@ -633,6 +811,15 @@ nce_result_t nceExecutorSynchronize(nce_executor_handle_t executor, void* hip_st
     const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) {
         executor->log->add(1, "synchronize failed: %s", hipGetErrorString(e));
+        return NCE_RESULT_ERROR_UNKNOWN;
+    }
+    if (executor->pk_host_error != nullptr && *executor->pk_host_error != 0) {
+        // A persistent segment gave up (a bounded wait ran out, or its workgroups were not placed as expected): what it
+        // wrote is incomplete. Persistent launches are off for this executor from here on; the caller re-enqueues.
+        executor->log->add(1, "a persistent task-list launch did not complete (code %u); its outputs are invalid, persistent launches are now off",
+                           *executor->pk_host_error);
+        *executor->pk_host_error = 0;
+        executor->pk_off.store(true);
         return NCE_RESULT_ERROR_UNKNOWN;
     }
     return NCE_RESULT_SUCCESS;

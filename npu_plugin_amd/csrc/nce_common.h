@@ -120,6 +120,8 @@ struct Options {
     int wres[4] = {0, 0, 0, 0};  // ... with these values
     int halo_tile = -1;       // NCE_HIP_CONV_TILE: force one halo tile shape (0..3)
     bool no_fuse = false;     // NCE_HIP_NO_FUSE: task lists never run a convolution and the add after it as one launch
+    int persistent = 0;       // NCE_HIP_PERSISTENT: task lists run runs of weights-resident convolutions as one persistent launch
+    int persistent_wait_us = 2000000;  // NCE_HIP_PERSISTENT_WAIT_US: time after which a persistent launch's waits give up
     int tiled = -1;           // NCE_HIP_CONV_TILED: -1 automatic, 0 never, 1.. force that shape of the LDS-tiled kernel
     bool env_path = false;    // NCE_HIP_CONV_PATH was given at all (switches the conv + add fusion off, as NO_FUSE does)
 };
@@ -130,6 +132,9 @@ struct RecordedLaunch {
     dim3 grid, block;
     uint32_t lds = 0;
     std::vector<uint64_t> arg;  // argument bytes (8-byte aligned storage; the largest member of every argument struct is 8 bytes)
+    int32_t tag = 0;            // weights-resident convolution kernels: their template parameters, packed (else 0)
+    void* clear = nullptr;      // device memory to zero on the stream before the launch (persistent segments: their counters)
+    uint32_t clear_bytes = 0;
 };
 
 // What a launch_* function needs besides its task: the executor's options and, when a task list prepares its
@@ -138,6 +143,9 @@ struct RecordedLaunch {
 struct LaunchContext {
     const Options* opt = nullptr;
     std::vector<RecordedLaunch>* record = nullptr;
+    // Per-XCD form: the task is one eighth of the batch, to be run by the 32 CUs of one XCD inside a persistent segment
+    // (grids are sized for 32 CUs; only the weights-resident convolution kernels take part).
+    bool per_xcd = false;
 };
 extern thread_local LaunchContext tls_launch;
 inline const Options& options() {
@@ -147,9 +155,10 @@ inline const Options& options() {
 
 // Launch `kernel(arg)` now, or record the launch when a task list is being prepared.
 template <typename Arg>
-inline hipError_t emit(void (*kernel)(Arg), dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Arg& arg) {
+inline hipError_t emit(void (*kernel)(Arg), dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Arg& arg, int tag = 0) {
     if (std::vector<RecordedLaunch>* rec = tls_launch.record) {
         RecordedLaunch r;
+        r.tag = tag;
         r.func = reinterpret_cast<const void*>(kernel);
         r.grid = grid;
         r.block = block;
@@ -162,7 +171,12 @@ inline hipError_t emit(void (*kernel)(Arg), dim3 grid, dim3 block, size_t lds, h
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, arg);
     return hipGetLastError();
 }
+// Zeroes device memory (16-byte granules) with a kernel on the stream.
+hipError_t pk_clear(void* p, uint32_t bytes, hipStream_t stream);
 inline hipError_t replay(const RecordedLaunch& r, hipStream_t stream) {
+    if (r.clear != nullptr) {
+        if (const hipError_t e = pk_clear(r.clear, r.clear_bytes, stream); e != hipSuccess) return e;
+    }
     void* args[1] = {const_cast<uint64_t*>(r.arg.data())};
     return hipLaunchKernel(r.func, r.grid, r.block, args, r.lds, stream);
 }

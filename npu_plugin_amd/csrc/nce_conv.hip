@@ -304,6 +304,7 @@ static bool overlaps(const TensorDev& x, const TensorDev& y) {
 
 // Which convolutions take the LDS-tiled kernel: 0 = none of its shapes, else the shape (0 within a forced value: automatic).
 static int tiled_shape_for(const ConvArgs& a) {
+    if (tls_launch.per_xcd) return 0;
     const int forced = options().tiled;
     if (forced >= 0) return forced;
     // Measured over the ResNet-50 layer shapes at batch 32, 128 and 512: the 128 x 128 tile is 10-15 % ahead of the
@@ -318,7 +319,7 @@ static int tiled_shape_for(const ConvArgs& a) {
 }
 
 hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskDev& add, const Box& ab, hipStream_t stream) {
-    if (options().no_fuse || options().env_path) return hipErrorNotSupported;
+    if (options().no_fuse || (options().env_path && !tls_launch.per_xcd)) return hipErrorNotSupported;
     const TensorDev& o = conv.out;
     const bool conv_full = cb.x0 == 0 && cb.y0 == 0 && cb.z0 == 0 && cb.bw == o.w && cb.bh == o.h && cb.bc == o.c;
     const bool add_full = ab.x0 == 0 && ab.y0 == 0 && ab.z0 == 0 && ab.bw == add.out.w && ab.bh == add.out.h && ab.bc == add.out.c;
@@ -359,6 +360,7 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     ConvArgs a;
     if (const hipError_t e0 = make_conv_args(t, box, a); e0 != hipSuccess) return e0;
     if (a.M == 0 || box.bc == 0) return hipSuccess;
+    if (tls_launch.per_xcd) return launch_conv_wres(a, stream, false);  // (nothing else takes part in persistent segments)
     // tuning and test knob: 1 = skip the weights-resident kernel, 2 = gather kernel only
     const int path = options().conv_path;
     // Reductions too long for one LDS slice: the halo kernel is the faster one for 3-wide kernels (measured on

@@ -28,8 +28,18 @@ inline FastDiv make_fastdiv(uint32_t d) {
     return f;
 }
 
-__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f) {
+// (F: FastDiv in any address space)
+template <typename F>
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const F& f) {
     return f.m == 0 ? n : (__umulhi(n, f.m) >> f.sh);
+}
+
+// A copy, in registers, of a struct that may live in the constant address space.
+template <typename T, typename S>
+__device__ __forceinline__ T generic_copy(const S& src) {
+    T t;
+    __builtin_memcpy(&t, &src, sizeof(T));
+    return t;
 }
 
 struct ConvArgs {

@@ -63,13 +63,15 @@ __device__ __forceinline__ EpiPack epi_pack_setup(const PpeF64& pu) {
 
 typedef unsigned short fz_u16x2 __attribute__((ext_vector_type(2)));
 
-template <int NF, int BF, int PMODE, bool FZ = false>
-__device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
+// (CA, FZP: ConvArgs and a pointer to FuseAdd, either of them possibly in the constant address space)
+template <int NF, int BF, int PMODE, bool FZ = false, typename CA, typename FZP = const FuseAdd*>
+__device__ __forceinline__ void wres_epilogue(const CA& a, const EpiSmem& s, const double* sBfull, const int32_t* sCorr,
                                               const v4i (&acc)[NF][BF], const int32_t (&dws)[BF], int q, int noc,
                                               uint8_t* const (&dst)[BF], const bool (&valid)[BF], const PpeF64& pu,
-                                              const EpiPack& ep, const FuseAdd* fz = nullptr, const uint4* other = nullptr) {
+                                              const EpiPack& ep, FZP fz = nullptr, const uint4* other = nullptr) {
     const int ch0 = 4 * NF * q;
     if (ch0 >= noc) return;
+    const PpeDev ppe_args = generic_copy<PpeDev>(a.ppe);
     static_assert(!FZ || NF == 4, "fused add: a lane holds 16 channels");
     uint32_t wo[BF][NF];
 #pragma unroll
@@ -99,7 +101,7 @@ __device__ __forceinline__ void wres_epilogue(const ConvArgs& a, const EpiSmem& 
             for (int x = 0; x < BF; ++x) {
                 const int32_t av = acc[f][x][r] + dws[x];  // (+ dw * sum of the pixel's activations; 0 when dw == 0)
                 if (PMODE == PPE_MODE_INT) {
-                    const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), a.ppe);
+                    const int32_t y = ppe_apply((int32_t)((uint32_t)av + (uint32_t)corr), bias, table_mult(w2), table_shift(w2), ppe_args);
                     wo[x][f] |= ((uint32_t)y & 0xFFu) << (8 * r);
                 } else if (PMODE == PPE_MODE_HI) {
                     // y = floor(((av + bias') * mult + 2^(shift-1) + zp * 2^shift) / 2^shift), everything scaled

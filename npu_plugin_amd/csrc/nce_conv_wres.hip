@@ -22,6 +22,7 @@
 // 64 a step never straddles taps and the tap bookkeeping is scalar; other channel counts take the
 // per-lane path (template MODE 2). Semantics and the fused PPE are the ones of nce_conv.hip.
 #include "nce_conv_epi.h"
+#include "nce_conv_pk.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -51,9 +52,9 @@ struct WresArgs {
     int32_t fused;      // host: the launch must carry the add in fz (or fail with hipErrorNotSupported)
 };
 
-// This file is compiled three times (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
+// This file is compiled four times (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
 // the 32-channel kernels and the chunked kernel, WRES_PART 1 the 64-channel kernels with 16- and 32-pixel tiles behind this
-// entry point, WRES_PART 2 those with 64-pixel tiles.
+// entry point, WRES_PART 2 those with 64-pixel tiles, WRES_PART 3 the persistent form (nce_conv_pk.h).
 #ifndef WRES_PART
 #define WRES_PART 0
 #endif
@@ -90,8 +91,38 @@ constexpr int kMaxSteps = 80;  // 144 KiB / (2 fragments * 1 KiB) = 72 steps, pa
 // the constant joins the per-channel constants.
 // LM packs the three flags: 0 plain, 1 TRL, 2 TBL, 3 plain + ASUM, 4 TRL + ASUM.
 enum { LM_PLAIN = 0, LM_TRL = 1, LM_TBL = 2, LM_PLAIN_ASUM = 3, LM_TRL_ASUM = 4, LM_PLAIN_FZ = 5 };  // 5: plain + fused residual add
-template <int NF, int BF, int MODE, int D, int LM>
-__global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
+// The workgroup's LDS tables besides the staged weights.
+template <int OCT, int NSTEP>
+struct WresSmem {
+    int32_t sW2[OCT], sBias[OCT];
+    double sM[OCT], sBc[OCT], sMd[OCT];  // scale, bias term, scale * da
+    // Weight sums: every wave leaves the partial sums of the fragments it staged in its row of sWpart; after
+    // the barrier every wave folds the total into its OWN copy of the per-channel constants, so that no
+    // second barrier is needed.
+    int32_t sWpart[8][OCT];
+    int32_t sCorr[8][OCT];   // integer path: da * sum of weights
+    double sBfull[8][OCT];   // FP64 paths: bias term + da * M * sum of weights (+ output zero point)
+    int32_t sFlags;
+    StepEntry sStep[NSTEP];  // per-lane mode: one entry per 16-byte unit
+};
+template <int NF, int MODE>
+using WresSmemOf = WresSmem<16 * NF, MODE == WRES_GENERIC ? 4 * kMaxSteps : kMaxSteps>;
+
+// No-op hook of the plain kernel (see conv_wres_body).
+struct NoInputWait {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// The work of one workgroup: pixel group `group` (of w.ngroups) of channel slice `slice`. sWt: the dynamic LDS for the
+// weights; sm: the tables. input_wait() is called by every wave, in uniform control flow, after the first weight requests
+// and before the first access to the input tensor: the persistent form of the kernel waits there for the layer that
+// produces the input (it may synchronise the workgroup).
+// WArgs: WresArgs, possibly qualified with the constant address space (the persistent form reads its arguments from a table
+// in memory; through that address space the compiler treats them as it treats kernel arguments - unchanging, fetched
+// where they are used).
+template <int NF, int BF, int MODE, int D, int LM, typename WArgs, typename InputWait>
+__device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t group, const uint32_t slice, uint8_t* const sWt,
+                                               WresSmemOf<NF, MODE>& sm, const InputWait& input_wait) {
     constexpr bool TRL = LM == LM_TRL || LM == LM_TRL_ASUM;
     constexpr bool TBL = LM == LM_TBL;
     constexpr bool ASUM = LM == LM_PLAIN_ASUM || LM == LM_TRL_ASUM;
@@ -102,19 +133,19 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     static_assert(NF == 2 || NF == 4, "channel fragments");
     static_assert(D >= 2 || !TRL, "the permute of the next step needs a second ring slot");
     static_assert(!(TRL && TBL) && !(TBL && MODE == WRES_GENERIC), "the step table serves the plain load order of modes 0 and 1");
-    const ConvArgs& a = w.a;
+    const auto& a = w.a;
+    const PpeDev ppe_args = generic_copy<PpeDev>(a.ppe);  // (for the helpers that take a reference)
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
-    __shared__ int32_t sW2[OCT], sBias[OCT];
-    __shared__ double sM[OCT], sBc[OCT], sMd[OCT];  // scale, bias term, scale * da
-    // Weight sums: every wave leaves the partial sums of the fragments it staged in its row of sWpart; after
-    // the barrier every wave folds the total into its OWN copy of the per-channel constants, so that no
-    // second barrier is needed.
-    __shared__ int32_t sWpart[8][OCT];
-    __shared__ int32_t sCorr[8][OCT];   // integer path: da * sum of weights
-    __shared__ double sBfull[8][OCT];   // FP64 paths: bias term + da * M * sum of weights (+ output zero point)
-    __shared__ int32_t sFlags;
-    __shared__ StepEntry sStep[MODE == WRES_GENERIC ? 4 * kMaxSteps : kMaxSteps];  // per-lane mode: one entry per 16-byte unit
+    auto& sW2 = sm.sW2;
+    auto& sBias = sm.sBias;
+    auto& sM = sm.sM;
+    auto& sBc = sm.sBc;
+    auto& sMd = sm.sMd;
+    auto& sWpart = sm.sWpart;
+    auto& sCorr = sm.sCorr;
+    auto& sBfull = sm.sBfull;
+    auto& sFlags = sm.sFlags;
+    auto& sStep = sm.sStep;
     const EpiSmem es = {sM, sBc, sW2, sBias, nullptr, nullptr};
 
     const int tid = threadIdx.x;
@@ -130,10 +161,8 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     const int kc = TRL ? kswz : lane >> 4;
     const int to_mfma = 4 * (4 * c16 + ((lane >> 4) ^ (2 * (c16 >> 3))));  // ds_bpermute source of lane 16k + p: piece k of pixel p
 
-    const int32_t oc0 = a.z0 + blockIdx.y * OCT;
+    const int32_t oc0 = a.z0 + (int32_t)slice * OCT;
     const int32_t noc = min(OCT, a.z0 + a.bc - oc0);
-    const uint32_t group = xcd_tile(blockIdx.x, w.ngroups);
-    if (group >= w.ngroups) return;  // uniform for the whole workgroup
 
     const int axor = (int)a.a_xor;
     const uint8_t* const fillp = &g_fill.b[(a.fill ^ a.a_xor) & 0xFFu][kc * 16];
@@ -389,6 +418,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
         // (No branch around these activation requests - the wait for the weights would otherwise have to cover
         // them too; a wave without a tile requests the last pixel's data, which setup() clamps to.)
         request(wave);
+        input_wait();
         setup();
         first_loads(false);
         if (consts_wave) do_consts();
@@ -414,7 +444,7 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
 
     const int flags = sFlags;
-    const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
+    const PpeF64 pu = ppe_f64_setup(ppe_args, (flags & 2) != 0);
     int pmode = ppe_mode_of(pu, (flags & 1) != 0);
     if (pmode == PPE_MODE_FOLDED && !(flags & 4)) pmode = PPE_MODE_HI;
     EpiPack ep = epi_pack_setup(pu);
@@ -565,6 +595,19 @@ __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
     }
 }
 
+template <int NF, int BF, int MODE, int D, int LM>
+__global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
+    __shared__ WresSmemOf<NF, MODE> sm;
+    const uint32_t group = xcd_tile(blockIdx.x, w.ngroups);
+    if (group >= w.ngroups) return;  // uniform for the whole workgroup
+    conv_wres_body<NF, BF, MODE, D, LM>(w, group, blockIdx.y, sWt, sm, NoInputWait{});
+}
+
+constexpr int wres_tag(int nf, int bf, int mode, int d, int lm) {
+    return nf * 10000 + bf * 1000 + mode * 100 + d * 10 + lm;
+}
+
 constexpr size_t kWresLdsCap = 144 * 1024;  // dynamic LDS one workgroup may take (160 KiB per CU less tables)
 
 template <int NF, int BF, int MODE, int D, int LM>
@@ -583,7 +626,8 @@ hipError_t launch_one(WresArgs& w, int nwaves, int tiles_per_wave, hipStream_t s
     auto kernel = &conv_wres_kernel<NF, BF, MODE, D, LM>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
-    return emit(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w);
+    // (the tag names the instantiation for the persistent form, which runs eight waves)
+    return emit(kernel, dim3(xcd_grid(w.ngroups), gy), dim3(64 * nwaves), lds, stream, w, nwaves == 8 ? wres_tag(NF, BF, MODE, D, LM) : 0);
 }
 
 template <int NF, int BF, int D>
@@ -1000,7 +1044,7 @@ hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, h
 hipError_t launch_wres_nf4_bf4(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t stream) {
     return launch_mode<4, 4>(w, mode, nwaves, tpw, stream);
 }
-#else
+#elif WRES_PART == 0
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse) {
     if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
@@ -1049,10 +1093,12 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     };
     const bool nf4_ok = wl4 <= kWresLdsCap && a.bc > 32;
     // (1x1 kernels over more than 64 input channels: measured faster with smaller pixel tiles, about 24 per CU)
-    const int64_t want = (w.ntaps == 1 && w.nsteps > 1) ? 6000 : 1500;
+    // (per-XCD form: an eighth of the work on an eighth of the CUs - the same choices as for the whole task)
+    const int cus = tls_launch.per_xcd ? 32 : 256;
+    const int64_t want = ((w.ntaps == 1 && w.nsteps > 1) ? 6000 : 1500) * cus / 256;
     int nf = nf4_ok ? 4 : 2, bf = 4;
     while (bf > 1 && wave_tiles(nf, bf) < want) bf >>= 1;
-    if (nf == 4 && wave_tiles(nf, bf) < 1500) nf = 2;
+    if (nf == 4 && wave_tiles(nf, bf) < 1500 * cus / 256) nf = 2;
     const int nwaves = 8;
     int tpw = 1;
     // Tiles per workgroup: one workgroup per CU where the tiles reach that far (the waves of a workgroup then
@@ -1060,7 +1106,7 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     const auto pick_tpg = [&](int nf_, int bf_, int nw_) {
         const int64_t ntiles = ((int64_t)a.M + 16 * bf_ - 1) / (16 * bf_);
         const int64_t slices = (a.bc + 16 * nf_ - 1) / (16 * nf_);
-        const int64_t groups = std::max<int64_t>(1, 256 / slices);
+        const int64_t groups = std::max<int64_t>(1, cus / slices);
         return (uint32_t)std::max<int64_t>(nw_, (ntiles + groups - 1) / groups);
     };
 
@@ -1079,5 +1125,160 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     return launch_bf<2>(w, bf, mode, nw, tpw, stream);
 }
 #endif  // WRES_PART
+
+#if WRES_PART == 3
+// ---- persistent segments (nce_conv_pk.h) ---------------------------------------------------------------------------------
+namespace {
+
+// The instantiations a segment may use: NF, BF, MODE, D, LM (those of the ResNet-50 bottleneck layers at 4 images per XCD).
+#define WRES_PK_VARIANTS(X)                                                                                           \
+    X(0, 4, 1, WRES_FAST, 4, LM_PLAIN) X(1, 4, 1, WRES_FAST, 4, LM_PLAIN_FZ) X(2, 4, 1, WRES_FAST_MASK, 4, LM_TRL)     \
+    X(4, 2, 1, WRES_FAST_MASK, 4, LM_TRL) X(5, 4, 2, WRES_FAST_MASK, 3, LM_TRL)  \
+    X(6, 4, 2, WRES_FAST, 2, LM_PLAIN_FZ) X(8, 2, 1, WRES_FAST, 4, LM_TRL)      \
+    X(10, 4, 2, WRES_FAST, 4, LM_PLAIN_FZ) X(11, 4, 2, WRES_FAST, 4, LM_PLAIN)     \
+    X(12, 4, 2, WRES_FAST, 2, LM_PLAIN)
+
+// Device table: [xcd][layer], the launch arguments of that XCD's share (pointers already advanced to its images).
+struct PkLayer {
+    int32_t variant;   // index in WRES_PK_VARIANTS
+    int32_t nvirt;     // workgroups' worth of work per XCD: pixel groups x channel slices
+    WresArgs w;
+};
+
+// Called by every wave of a workgroup before its first access to the layer's input: wait until all workgroups of the XCD
+// have finished the previous layer, then drop this CU's L1 lines (they may hold that layer's output buffer from its use
+// two layers ago). Bounded: a wait that runs out of time sets the error words and the workgroup leaves the kernel.
+struct PkInputWait {
+    PkCtl* ctl;
+    uint32_t* s_err;      // LDS
+    uint64_t deadline;    // wall clock ticks (100 MHz)
+    int32_t layer;        // wait for `layer - 1` (none for 0)
+    uint32_t xcd;
+    __device__ __forceinline__ void operator()() const {
+        if (layer == 0) return;
+        if (threadIdx.x == 0) {
+            const uint32_t* ctr = &ctl->arrive[(xcd * kPkMaxLayers + (layer - 1)) * 16];
+            while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)kPkPerXcd) {
+                __builtin_amdgcn_s_sleep(1);
+                if (wall_clock64() > deadline) {
+                    *s_err = 1;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        asm volatile("buffer_inv sc0" ::: "memory");
+    }
+};
+
+__global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];
+    __shared__ __attribute__((aligned(16))) uint8_t sm_raw[sizeof(WresSmemOf<4, WRES_FAST>)];  // (the largest of the variants' tables)
+    __shared__ uint32_t s_err;
+    // The table is read through the constant address space: it does not change while the kernel runs, and the compiler
+    // may then treat its fields like kernel arguments (fetched where they are used instead of kept or spilled).
+
+    const uint32_t xcd = blockIdx.x & 7u, rank = blockIdx.x >> 3;
+    const uint32_t xcc = (uint32_t)__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15u;  // HW_REG_XCC_ID
+    if (threadIdx.x == 0) s_err = xcc != xcd ? 2u : 0u;
+    __syncthreads();
+    const uint64_t deadline = wall_clock64() + (uint64_t)p.wait_us * 100ull;
+    for (int l = 0; l < p.nlayers; ++l) {
+        if (__builtin_amdgcn_readfirstlane(s_err) != 0) break;  // (uniform: read after a barrier)
+        typedef const __attribute__((address_space(4))) PkLayer* table_ptr_t;
+        const table_ptr_t L = (table_ptr_t)(uintptr_t)p.layers + (xcd * (uint32_t)p.nlayers + l);
+        const int32_t variant = L->variant, nvirt = L->nvirt;
+        const __attribute__((address_space(4))) WresArgs& w = L->w;
+        const PkInputWait wait = {p.ctl, &s_err, deadline, l, xcd};
+        for (uint32_t v = rank; v < (uint32_t)nvirt; v += kPkPerXcd) {
+            const uint32_t slice = v / w.ngroups, group = v - slice * w.ngroups;
+            switch (variant) {
+#define X(ID, NF, BF, MODE, D, LM)                                                                                        \
+    case ID:                                                                                                              \
+        conv_wres_body<NF, BF, MODE, D, LM>(w, group, slice, sWt, *reinterpret_cast<WresSmemOf<NF, MODE>*>(sm_raw), wait); \
+        break;
+                WRES_PK_VARIANTS(X)
+#undef X
+            default: break;
+            }
+            __syncthreads();  // every wave has left the LDS weights and tables
+        }
+        // this workgroup's share of layer l is stored: count it in
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (threadIdx.x == 0)
+            __hip_atomic_fetch_add(&p.ctl->arrive[(xcd * kPkMaxLayers + l) * 16], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && s_err != 0) {
+        atomicMax(&p.ctl->error, s_err);
+        if (p.host_error != nullptr) atomicMax(p.host_error, s_err);
+    }
+}
+
+// Zeroes a segment's counters ahead of its launch (a kernel rather than a memset node, so that a caller may capture the
+// list's launches into a graph).
+__global__ __launch_bounds__(256) void pk_clear_kernel(uint4* p, uint32_t n16) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+int pk_variant_of(int tag) {
+#define X(ID, NF, BF, MODE, D, LM) \
+    if (tag == wres_tag(NF, BF, MODE, D, LM)) return ID;
+    WRES_PK_VARIANTS(X)
+#undef X
+    return -1;
+}
+
+}  // namespace
+
+hipError_t pk_clear(void* p, uint32_t bytes, hipStream_t stream) {
+    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(p) % 16 != 0) return hipErrorInvalidValue;
+    const uint32_t n16 = bytes / 16;
+    if (n16 == 0) return hipSuccess;
+    hipLaunchKernelGGL(pk_clear_kernel, dim3((n16 + 255) / 256), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
+    return hipGetLastError();
+}
+
+bool wres_pk_has_variant(int tag) {
+    return pk_variant_of(tag) >= 0;
+}
+
+hipError_t wres_pk_make(const std::vector<PkLayerDesc>& layers, std::vector<uint8_t>* table, RecordedLaunch* launch) {
+    if (layers.empty() || (int)layers.size() > kPkMaxLayers) return hipErrorInvalidValue;
+    table->assign(8 * layers.size() * sizeof(PkLayer), 0);
+    size_t lds = 0;
+    for (size_t i = 0; i < layers.size(); ++i) {
+        const RecordedLaunch& r = *layers[i].launch;
+        PkLayer L;
+        memset(&L, 0, sizeof(L));
+        L.variant = pk_variant_of(r.tag);
+        if (L.variant < 0 || r.arg.size() * 8 < sizeof(WresArgs) || r.block.x != 512) return hipErrorNotSupported;
+        memcpy(&L.w, r.arg.data(), sizeof(WresArgs));
+        L.nvirt = (int32_t)(L.w.ngroups * r.grid.y);
+        for (int x = 0; x < 8; ++x) {
+            PkLayer Lx = L;
+            Lx.w.a.in += x * layers[i].d_in;
+            Lx.w.a.out += x * layers[i].d_out;
+            if (Lx.w.fz.other != nullptr) Lx.w.fz.other += x * layers[i].d_other;
+            if (Lx.w.fz.out != nullptr) Lx.w.fz.out += x * layers[i].d_fzout;
+            memcpy(table->data() + ((size_t)x * layers.size() + i) * sizeof(PkLayer), &Lx, sizeof(Lx));
+        }
+        lds = std::max<size_t>(lds, r.lds);
+    }
+    // (at least 100 KiB of dynamic LDS: no second workgroup fits a CU, so the 256 workgroups are one per CU)
+    lds = std::max<size_t>(lds, 100 * 1024);
+    auto kernel = &conv_wres_persistent_kernel;
+    static LdsGrant grant;
+    if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
+    launch->func = reinterpret_cast<const void*>(kernel);
+    launch->grid = dim3(kPkWorkgroups);
+    launch->block = dim3(512);
+    launch->lds = (uint32_t)lds;
+    launch->tag = 0;
+    return hipSuccess;
+}
+#endif  // WRES_PART == 3
 
 }  // namespace nce
