@@ -184,6 +184,18 @@ nce_result_t nceClusterTaskEnqueue(nce_executor_handle_t executor, const nce_clu
 nce_result_t nceTaskListCreate(nce_executor_handle_t executor, nce_task_list_handle_t* list);
 nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_task_desc_t* task);
 nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream);
+/* nceTaskListEnqueue for callers that cannot allocate device memory (code under stream capture, tight serving loops,
+ * harnesses that forbid hipMalloc). It has no counterpart in the reference. It runs the list the way nceTaskListEnqueue
+ * does for an executor created under NCE_HIP_PERSISTENT=1 - runs of consecutive weights-resident convolutions as one
+ * persistent launch each - but keeps those launches' layer tables, counters and error word in a fixed array in device
+ * memory that belongs to the library (281 KiB per GPU, held until the process ends) instead of allocating them, and
+ * calls neither hipMalloc nor hipFree. Limits: the persistent launches of one list may cover at most 64 layers together
+ * (more: NCE_RESULT_ERROR_UNSUPPORTED, nothing is launched); a list that nceTaskListEnqueue has prepared with device
+ * allocations is refused (NCE_RESULT_ERROR_INVALID_ARGUMENT). Every call on a GPU shares that GPU's array: calls whose
+ * launches may overlap on the GPU (two streams, two executors, two processes do not share it) race and must be
+ * serialised by the caller. Failures of a persistent launch are reported by nceExecutorSynchronize, as for
+ * nceTaskListEnqueue. */
+nce_result_t nceTaskListEnqueueNoAlloc(nce_task_list_handle_t list, void* hip_stream);
 nce_result_t nceTaskListDestroy(nce_task_list_handle_t list);
 
 /* Wait for everything this executor enqueued on the null stream / the given stream. */

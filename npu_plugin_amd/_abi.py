@@ -195,6 +195,7 @@ SYMBOLS = {
     "nceTaskListCreate": (C.c_int, [C.c_void_p, _P(C.c_void_p)]),
     "nceTaskListAppend": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc)]),
     "nceTaskListEnqueue": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "nceTaskListEnqueueNoAlloc": (C.c_int, [C.c_void_p, C.c_void_p]),
     "nceTaskListDestroy": (C.c_int, [C.c_void_p]),
     "nceExecutorSynchronize": (C.c_int, [C.c_void_p, C.c_void_p]),
     "nceLogHandleGetString": (C.c_int, [C.c_void_p, _P(C.c_size_t), C.c_char_p]),

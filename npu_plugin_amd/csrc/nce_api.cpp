@@ -23,6 +23,10 @@ struct nce_executor_s {
     // synchronise; persistent launches are then switched off for this executor).
     uint32_t* pk_host_error = nullptr;
     std::atomic<bool> pk_off{false};
+    // The library's fixed workspace on this executor's device (looked up at creation), for nceTaskListEnqueueNoAlloc.
+    nce::PkWorkspace ws;
+    bool ws_ok = false;
+    std::atomic<bool> ws_used{false};   // a launch that reports through ws.error may be in flight
     ~nce_executor_s() {
         if (pk_host_error != nullptr) (void)hipHostFree(pk_host_error);
     }
@@ -458,14 +462,18 @@ struct nce_task_list_s {
     std::mutex mu;
     std::vector<Plan> plans;
     std::vector<nce::RecordedLaunch> launches;
-    std::vector<void*> device_mem;  // tables and counters of persistent segments
+    std::vector<void*> device_mem;  // tables and counters of persistent segments (none in the fixed-workspace form)
+    std::vector<uint8_t> ws_table;  // fixed-workspace form: the segments' tables, copied to the workspace by every enqueue
     bool prepared = false;
+    bool fixed_ws = false;          // prepared for the fixed workspace
     bool has_segments = false;
     void drop_prepared() {
         for (void* p : device_mem) (void)hipFree(p);
         device_mem.clear();
+        ws_table.clear();
         launches.clear();
         prepared = false;
+        fixed_ws = false;
         has_segments = false;
     }
     ~nce_task_list_s() { drop_prepared(); }
@@ -577,12 +585,14 @@ nce_result_t run_plans(nce_executor_s* ex, const std::vector<Plan>& plans, hipSt
 }
 
 // Replace every run of two or more consecutive launches that have a per-XCD form (and whose tensors allow it) by one
-// persistent launch. Allocates the segments' device tables and counters (kept in list->device_mem).
-nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts) {
+// persistent launch. Allocates the segments' device tables and counters (kept in list->device_mem) - or, with fixed_ws,
+// allocates nothing: the tables are gathered in list->ws_table for the executor's fixed workspace, whose counters and error
+// word the launches use.
+nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, bool fixed_ws) {
     nce_executor_s* const ex = list->ex;
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, ex->device) != hipSuccess || prop.multiProcessorCount != nce::kPkWorkgroups) return NCE_RESULT_SUCCESS;
-    if (ex->pk_host_error == nullptr) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ex->device) != hipSuccess || cus != nce::kPkWorkgroups) return NCE_RESULT_SUCCESS;
+    if (!fixed_ws && ex->pk_host_error == nullptr) {
         if (hipHostMalloc(reinterpret_cast<void**>(&ex->pk_host_error), 64, hipHostMallocDefault) != hipSuccess) return NCE_RESULT_SUCCESS;
         *ex->pk_host_error = 0;
     }
@@ -613,6 +623,29 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts) {
         const hipError_t e = nce::wres_pk_make(layers, &table, &seg);
         void* d_table = nullptr;
         void* d_ctl = nullptr;
+        if (fixed_ws && e == hipSuccess) {
+            if (list->ws_table.size() + table.size() > ex->ws.table_bytes) {
+                ex->log->add(1, "task list: its persistent launches cover more than %d layers, the limit of the fixed workspace "
+                                "(nceTaskListEnqueueNoAlloc); use nceTaskListEnqueue or a shorter list", nce::kPkMaxLayers);
+                return NCE_RESULT_ERROR_UNSUPPORTED;
+            }
+            nce::PkArgs args;
+            args.layers = ex->ws.table + list->ws_table.size();
+            args.ctl = ex->ws.ctl;
+            args.host_error = ex->ws.error;
+            args.nlayers = (int32_t)(j - i);
+            args.wait_us = (uint32_t)ex->opt.persistent_wait_us;
+            list->ws_table.insert(list->ws_table.end(), table.begin(), table.end());
+            seg.arg.resize((sizeof(args) + 7) / 8);
+            memcpy(seg.arg.data(), &args, sizeof(args));
+            seg.clear = ex->ws.ctl;
+            seg.clear_bytes = (uint32_t)sizeof(nce::PkCtl);
+            out.push_back(std::move(seg));
+            list->has_segments = true;
+            ex->log->add(3, "task list: launches %zu..%zu run as one persistent launch (fixed workspace)", i, j - 1);
+            i = j;
+            continue;
+        }
         if (e != hipSuccess || hipMalloc(&d_table, table.size()) != hipSuccess) {
             for (size_t k = i; k < j; ++k) out.push_back(std::move(list->launches[k]));
             i = j;
@@ -680,6 +713,12 @@ nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* 
             delete ex;
             delete lg;
             return NCE_RESULT_ERROR_UNSUPPORTED;
+        }
+        // The fixed workspace's address on this device (nceTaskListEnqueueNoAlloc); everything else works without it.
+        if (hipSetDevice(desc.device_id) == hipSuccess) {
+            const hipError_t we = nce::pk_workspace(desc.device_id, &ex->ws);
+            ex->ws_ok = we == hipSuccess;
+            if (!ex->ws_ok) lg->add(2, "fixed workspace not available on device %d: %s", desc.device_id, hipGetErrorString(we));
         }
     }
     *executor = ex;
@@ -752,41 +791,68 @@ nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_ta
     }
 }
 
-nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
+namespace {
+
+// Both enqueue forms. fixed_ws: nothing may be allocated or freed on the device - persistent segments (always tried in that
+// form) keep their tables, counters and error word in the executor's fixed workspace.
+nce_result_t enqueue_list(nce_task_list_handle_t list, void* hip_stream, bool fixed_ws) {
     if (list == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
-    if (list->ex->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
-    if (hipSetDevice(list->ex->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
+    nce_executor_s* const ex = list->ex;
+    if (ex->device < 0) return NCE_RESULT_ERROR_UNSUPPORTED;
+    if (hipSetDevice(ex->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     try {
         std::lock_guard<std::mutex> lk(list->mu);
-        if (list->prepared && list->has_segments && list->ex->pk_off.load()) list->drop_prepared();
+        if (fixed_ws && !ex->ws_ok) {
+            ex->log->add(1, "nceTaskListEnqueueNoAlloc: the fixed workspace was not found on device %d when the executor was created", ex->device);
+            return NCE_RESULT_ERROR_UNSUPPORTED;
+        }
+        if (list->prepared && list->fixed_ws != fixed_ws) {
+            if (fixed_ws && !list->device_mem.empty()) {
+                // (switching forms would have to free what nceTaskListEnqueue allocated for this list)
+                ex->log->add(1, "nceTaskListEnqueueNoAlloc: this list holds device allocations made by nceTaskListEnqueue; use one form per list");
+                return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+            }
+            list->drop_prepared();
+        }
+        if (list->prepared && list->has_segments && ex->pk_off.load()) list->drop_prepared();  // (the fixed form holds no device memory)
         if (!list->prepared) {
             // Kernel choice, grids and argument blocks are worked out once, here; later calls only replay them.
             list->drop_prepared();
-            const bool persistent = list->ex->opt.persistent != 0 && !list->ex->pk_off.load();
+            const bool persistent = (fixed_ws || ex->opt.persistent != 0) && !ex->pk_off.load();
             std::vector<PkAlt> alts;
             {
-                const ScopedLaunch ctx(&list->ex->opt, &list->launches);
-                const nce_result_t r = run_plans(list->ex, list->plans, nullptr, persistent ? &alts : nullptr);
+                const ScopedLaunch ctx(&ex->opt, &list->launches);
+                const nce_result_t r = run_plans(ex, list->plans, nullptr, persistent ? &alts : nullptr);
                 if (r != NCE_RESULT_SUCCESS) {
                     list->launches.clear();
                     return r;
                 }
             }
             if (persistent) {
-                const ScopedLaunch ctx(&list->ex->opt, nullptr);
-                const nce_result_t r = build_segments(list, alts);
+                const ScopedLaunch ctx(&ex->opt, nullptr);
+                const nce_result_t r = build_segments(list, alts, fixed_ws);
                 if (r != NCE_RESULT_SUCCESS) {
                     list->drop_prepared();
                     return r;
                 }
             }
+            list->fixed_ws = fixed_ws;
             list->prepared = true;
+        }
+        if (list->fixed_ws && list->has_segments) {
+            // The workspace holds whatever the last list to use it left there: this list's tables go in ahead of its launches.
+            const hipError_t e = hipMemcpyAsync(ex->ws.table, list->ws_table.data(), list->ws_table.size(), hipMemcpyHostToDevice, stream);
+            if (e != hipSuccess) {
+                ex->log->add(1, "copy of the layer tables to the fixed workspace failed: %s", hipGetErrorString(e));
+                return NCE_RESULT_ERROR_UNKNOWN;
+            }
+            ex->ws_used.store(true);
         }
         for (const nce::RecordedLaunch& l : list->launches) {
             const hipError_t e = nce::replay(l, stream);
             if (e != hipSuccess) {
-                list->ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
+                ex->log->add(1, "kernel launch failed: %s", hipGetErrorString(e));
                 return NCE_RESULT_ERROR_UNKNOWN;
             }
         }
@@ -796,6 +862,16 @@ nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
     } catch (...) {
         return NCE_RESULT_ERROR_UNKNOWN;
     }
+}
+
+}  // namespace
+
+nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream) {
+    return enqueue_list(list, hip_stream, false);
+}
+
+nce_result_t nceTaskListEnqueueNoAlloc(nce_task_list_handle_t list, void* hip_stream) {
+    return enqueue_list(list, hip_stream, true);
 }
 
 nce_result_t nceTaskListDestroy(nce_task_list_handle_t list) {
@@ -813,12 +889,22 @@ nce_result_t nceExecutorSynchronize(nce_executor_handle_t executor, void* hip_st
         executor->log->add(1, "synchronize failed: %s", hipGetErrorString(e));
         return NCE_RESULT_ERROR_UNKNOWN;
     }
+    uint32_t code = 0;
     if (executor->pk_host_error != nullptr && *executor->pk_host_error != 0) {
+        code = *executor->pk_host_error;
+        *executor->pk_host_error = 0;
+    }
+    if (executor->ws_used.load()) {  // (the fixed workspace's error word lives in device memory)
+        uint32_t ws_code = 0;
+        if (hipMemcpy(&ws_code, executor->ws.error, sizeof(ws_code), hipMemcpyDeviceToHost) == hipSuccess && ws_code != 0) {
+            (void)hipMemset(executor->ws.error, 0, sizeof(ws_code));
+            code = std::max(code, ws_code);
+        }
+    }
+    if (code != 0) {
         // A persistent segment gave up (a bounded wait ran out, or its workgroups were not placed as expected): what it
         // wrote is incomplete. Persistent launches are off for this executor from here on; the caller re-enqueues.
-        executor->log->add(1, "a persistent task-list launch did not complete (code %u); its outputs are invalid, persistent launches are now off",
-                           *executor->pk_host_error);
-        *executor->pk_host_error = 0;
+        executor->log->add(1, "a persistent task-list launch did not complete (code %u); its outputs are invalid, persistent launches are now off", code);
         executor->pk_off.store(true);
         return NCE_RESULT_ERROR_UNKNOWN;
     }

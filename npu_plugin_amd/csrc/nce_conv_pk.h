@@ -38,6 +38,17 @@ struct PkLayerDesc {
     int64_t d_in, d_out, d_other, d_fzout;
 };
 
+// The library's fixed workspace on a device: what a segment otherwise gets from hipMalloc, for the enqueue form that
+// allocates nothing. One per device and process, shared by every list that uses that form.
+struct PkWorkspace {
+    uint32_t* error = nullptr;   // sticky error word (device memory): raised by a segment that gave up, cleared by the host
+    PkCtl* ctl = nullptr;        // counters, zeroed before every segment
+    uint8_t* table = nullptr;    // layer tables of the list that is running
+    size_t table_bytes = 0;      // room for the tables of kPkMaxLayers layers
+};
+// Looks the workspace's device address up (once per device, cached). `device` must be the calling thread's current device.
+hipError_t pk_workspace(int device, PkWorkspace* ws);
+
 bool wres_pk_has_variant(int tag);
 // The device table of a segment (to be uploaded) and its launch: kernel, grid, block, LDS size; the argument block
 // (PkArgs) is filled in by the caller once the table and counters have device addresses.

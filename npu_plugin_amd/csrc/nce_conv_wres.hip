@@ -24,6 +24,7 @@
 #include "nce_conv_epi.h"
 #include "nce_conv_pk.h"
 
+#include <mutex>
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
@@ -1223,6 +1224,16 @@ __global__ __launch_bounds__(256) void pk_clear_kernel(uint4* p, uint32_t n16) {
     if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
 }
 
+// ---- fixed workspace -----------------------------------------------------------------------------------------------------
+// Layout: [0, 256) the sticky error word; then the counters; then the layer tables of up to kPkMaxLayers layers.
+constexpr size_t kWsCtl = 256;
+constexpr size_t kWsTable = kWsCtl + (sizeof(PkCtl) + 255) / 256 * 256;
+constexpr size_t kWsTableBytes = (size_t)8 * kPkMaxLayers * sizeof(PkLayer);
+constexpr size_t kWsBytes = kWsTable + kWsTableBytes;   // 281 KiB on every device the library runs on
+// Host code must never use this name as an address (on the host it is a stand-in, not device memory): the device
+// address comes from hipGetSymbolAddress, below, and only that pointer is handed to kernels and copies.
+static __device__ __align__(256) uint8_t scratch[kWsBytes];
+
 int pk_variant_of(int tag) {
 #define X(ID, NF, BF, MODE, D, LM) \
     if (tag == wres_tag(NF, BF, MODE, D, LM)) return ID;
@@ -1239,6 +1250,29 @@ hipError_t pk_clear(void* p, uint32_t bytes, hipStream_t stream) {
     if (n16 == 0) return hipSuccess;
     hipLaunchKernelGGL(pk_clear_kernel, dim3((n16 + 255) / 256), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
     return hipGetLastError();
+}
+
+hipError_t pk_workspace(int device, PkWorkspace* ws) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static uint8_t* base_of[kMaxDevices] = {};
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    int current = -1;
+    if (const hipError_t e = hipGetDevice(&current); e != hipSuccess) return e;
+    if (current != device) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lk(mu);
+    if (base_of[device] == nullptr) {
+        void* p = nullptr;
+        if (const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        base_of[device] = static_cast<uint8_t*>(p);
+    }
+    uint8_t* const base = base_of[device];
+    ws->error = reinterpret_cast<uint32_t*>(base);
+    ws->ctl = reinterpret_cast<PkCtl*>(base + kWsCtl);
+    ws->table = base + kWsTable;
+    ws->table_bytes = kWsTableBytes;
+    return hipSuccess;
 }
 
 bool wres_pk_has_variant(int tag) {

@@ -176,6 +176,10 @@ class TaskList:
     def enqueue(self, stream=None):
         self._ex._check(self._lib.nceTaskListEnqueue(self._h, C.c_void_p(stream or 0)))
 
+    def enqueue_no_alloc(self, stream=None):
+        """nceTaskListEnqueueNoAlloc: the same launches with no device allocation (the library's fixed workspace)."""
+        self._ex._check(self._lib.nceTaskListEnqueueNoAlloc(self._h, C.c_void_p(stream or 0)))
+
     def destroy(self):
         if self._h:
             self._lib.nceTaskListDestroy(self._h)
