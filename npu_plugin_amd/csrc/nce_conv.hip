@@ -307,15 +307,22 @@ static int tiled_shape_for(const ConvArgs& a) {
     if (tls_launch.per_xcd) return 0;
     const int forced = options().tiled;
     if (forced >= 0) return forced;
-    // Measured over the ResNet-50 layer shapes at batch 32, 128 and 512: the 128 x 128 tile is 10-15 % ahead of the
-    // weights-resident kernels for long reductions over many output channels while its grid gives every CU two to four
-    // workgroups; with fewer it leaves CUs idle, with more the weights-resident kernels amortise their staging over many
-    // tiles per workgroup and win again.
-    if (a.IC % 64 != 0 || a.dw != 0 || (int64_t)a.KY * a.KX * a.IC < 1024 || a.bc < 256) return 0;
+    // Measured over the ResNet-50 layer shapes at batch 32, 128 and 256 against the weights-resident kernels. The 128 x 128
+    // tile with steps of 128 bytes of the reduction (one barrier and one LDS round trip per 32 matrix instructions of a
+    // wave; input channels a multiple of 128) is 3-25 % ahead - 45 % for 3x3 over 512 channels - where the reduction is long
+    // and the output channels many: from 1024 bytes of reduction for 256 channels or more once there are ~200 workgroups
+    // (fewer leave CUs idle), for 128 channels from 384 workgroups; from 512 bytes only for grids of 384 workgroups or more
+    // and not for 256 channels over very many pixels, where the weights-resident kernels amortise their staging over many
+    // tiles per workgroup and win again. Shorter reductions and fewer channels always lose. The 64-byte-step shape (input
+    // channels not a multiple of 128) is 9 % slower and keeps the narrower window it was measured in.
+    const int64_t k = (int64_t)a.KY * a.KX * a.IC;
+    if (a.IC % 64 != 0 || a.dw != 0 || k < 512 || a.bc < 128) return 0;
     const int64_t groups = (((int64_t)a.M + 127) / 128) * ((a.bc + 127) / 128);
-    // (steps of 128 bytes of the reduction - one barrier and one LDS round trip per 32 matrix instructions of a wave - where
-    // the input channels allow: measured 9 % ahead of 64-byte steps)
-    return groups >= 384 && groups <= 1024 ? (a.IC % 128 == 0 ? 5 : 1) : 0;
+    if (a.IC % 128 != 0) return k >= 1024 && a.bc >= 256 && groups >= 384 && groups <= 1024 ? 1 : 0;
+    bool use;
+    if (k >= 1024) use = a.bc >= 256 ? groups >= 200 : groups >= 384;
+    else use = a.bc >= 256 && groups >= 384 && (a.bc >= 512 || groups <= 1024);
+    return use ? 5 : 0;
 }
 
 hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskDev& add, const Box& ab, hipStream_t stream) {
