@@ -638,8 +638,6 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, boo
             list->ws_table.insert(list->ws_table.end(), table.begin(), table.end());
             seg.arg.resize((sizeof(args) + 7) / 8);
             memcpy(seg.arg.data(), &args, sizeof(args));
-            seg.clear = ex->ws.ctl;
-            seg.clear_bytes = (uint32_t)sizeof(nce::PkCtl);
             out.push_back(std::move(seg));
             list->has_segments = true;
             ex->log->add(3, "task list: launches %zu..%zu run as one persistent launch (fixed workspace)", i, j - 1);
@@ -652,7 +650,7 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, boo
             continue;
         }
         list->device_mem.push_back(d_table);
-        if (hipMalloc(&d_ctl, sizeof(nce::PkCtl)) != hipSuccess || hipMemcpy(d_table, table.data(), table.size(), hipMemcpyHostToDevice) != hipSuccess) {
+        if (hipMalloc(&d_ctl, sizeof(nce::PkCtl)) != hipSuccess || hipMemset(d_ctl, 0, sizeof(nce::PkCtl)) != hipSuccess || hipMemcpy(d_table, table.data(), table.size(), hipMemcpyHostToDevice) != hipSuccess) {
             for (size_t k = i; k < j; ++k) out.push_back(std::move(list->launches[k]));
             i = j;
             continue;
@@ -666,8 +664,6 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, boo
         args.wait_us = (uint32_t)ex->opt.persistent_wait_us;
         seg.arg.resize((sizeof(args) + 7) / 8);
         memcpy(seg.arg.data(), &args, sizeof(args));
-        seg.clear = d_ctl;
-        seg.clear_bytes = (uint32_t)sizeof(nce::PkCtl);
         out.push_back(std::move(seg));
         list->has_segments = true;
         ex->log->add(3, "task list: launches %zu..%zu run as one persistent launch", i, j - 1);
@@ -897,7 +893,9 @@ nce_result_t nceExecutorSynchronize(nce_executor_handle_t executor, void* hip_st
     if (executor->ws_used.load()) {  // (the fixed workspace's error word lives in device memory)
         uint32_t ws_code = 0;
         if (hipMemcpy(&ws_code, executor->ws.error, sizeof(ws_code), hipMemcpyDeviceToHost) == hipSuccess && ws_code != 0) {
+            // (a launch that gave up leaves the workspace's counters between multiples of 32)
             (void)hipMemset(executor->ws.error, 0, sizeof(ws_code));
+            (void)hipMemset(executor->ws.ctl, 0, sizeof(nce::PkCtl));
             code = std::max(code, ws_code);
         }
     }

@@ -133,8 +133,6 @@ struct RecordedLaunch {
     uint32_t lds = 0;
     std::vector<uint64_t> arg;  // argument bytes (8-byte aligned storage; the largest member of every argument struct is 8 bytes)
     int32_t tag = 0;            // weights-resident convolution kernels: their template parameters, packed (else 0)
-    void* clear = nullptr;      // device memory to zero on the stream before the launch (persistent segments: their counters)
-    uint32_t clear_bytes = 0;
 };
 
 // What a launch_* function needs besides its task: the executor's options and, when a task list prepares its
@@ -171,12 +169,7 @@ inline hipError_t emit(void (*kernel)(Arg), dim3 grid, dim3 block, size_t lds, h
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, arg);
     return hipGetLastError();
 }
-// Zeroes device memory (16-byte granules) with a kernel on the stream.
-hipError_t pk_clear(void* p, uint32_t bytes, hipStream_t stream);
 inline hipError_t replay(const RecordedLaunch& r, hipStream_t stream) {
-    if (r.clear != nullptr) {
-        if (const hipError_t e = pk_clear(r.clear, r.clear_bytes, stream); e != hipSuccess) return e;
-    }
     void* args[1] = {const_cast<uint64_t*>(r.arg.data())};
     return hipLaunchKernel(r.func, r.grid, r.block, args, r.lds, stream);
 }

@@ -21,12 +21,12 @@ constexpr int kPkPerXcd = 32;
 struct PkCtl {
     uint32_t error;                            // 1: a wait ran out of time, 2: a workgroup found itself on an unexpected XCD
     uint32_t pad[15];
-    uint32_t arrive[8 * kPkMaxLayers * 16];    // [xcd][layer], one 64-byte line per counter
+    uint32_t arrive[8 * kPkMaxLayers * 16];    // [xcd][layer], one 64-byte line per counter; multiples of 32 between launches
 };
 
 struct PkArgs {
     const void* layers;     // device table made by wres_pk_make
-    PkCtl* ctl;             // zeroed before every launch
+    PkCtl* ctl;             // counters: zero when first used, then only ever counted up (by 32 per launch and counter)
     uint32_t* host_error;   // host-visible word that receives ctl->error (may be null)
     int32_t nlayers;
     uint32_t wait_us;       // from the kernel's start; a wait still unsatisfied then gives up and the workgroup leaves
@@ -42,7 +42,7 @@ struct PkLayerDesc {
 // allocates nothing. One per device and process, shared by every list that uses that form.
 struct PkWorkspace {
     uint32_t* error = nullptr;   // sticky error word (device memory): raised by a segment that gave up, cleared by the host
-    PkCtl* ctl = nullptr;        // counters, zeroed before every segment
+    PkCtl* ctl = nullptr;        // counters (zero at load; zeroed again by the host after a launch that gave up)
     uint8_t* table = nullptr;    // layer tables of the list that is running
     size_t table_bytes = 0;      // room for the tables of kPkMaxLayers layers
 };

@@ -1155,11 +1155,13 @@ struct PkInputWait {
     uint64_t deadline;    // wall clock ticks (100 MHz)
     int32_t layer;        // wait for `layer - 1` (none for 0)
     uint32_t xcd;
+    uint32_t target;      // value the counter of `layer - 1` reaches when all workgroups of the XCD have arrived (thread 0)
     __device__ __forceinline__ void operator()() const {
         if (layer == 0) return;
         if (threadIdx.x == 0) {
             const uint32_t* ctr = &ctl->arrive[(xcd * kPkMaxLayers + (layer - 1)) * 16];
-            while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)kPkPerXcd) {
+            // (the counters are never reset and may wrap: compare by difference)
+            while ((int32_t)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
                 __builtin_amdgcn_s_sleep(1);
                 if (wall_clock64() > deadline) {
                     *s_err = 1;
@@ -1184,13 +1186,17 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
     if (threadIdx.x == 0) s_err = xcc != xcd ? 2u : 0u;
     __syncthreads();
     const uint64_t deadline = wall_clock64() + (uint64_t)p.wait_us * 100ull;
+    // The counters are not cleared between launches: every launch adds kPkPerXcd to each, so the value a counter must reach
+    // follows from what this workgroup's own arrival found there (launches that share counters run one after the other,
+    // and at most kPkPerXcd - 1 others can have arrived before this one).
+    uint32_t target = 0;
     for (int l = 0; l < p.nlayers; ++l) {
         if (__builtin_amdgcn_readfirstlane(s_err) != 0) break;  // (uniform: read after a barrier)
         typedef const __attribute__((address_space(4))) PkLayer* table_ptr_t;
         const table_ptr_t L = (table_ptr_t)(uintptr_t)p.layers + (xcd * (uint32_t)p.nlayers + l);
         const int32_t variant = L->variant, nvirt = L->nvirt;
         const __attribute__((address_space(4))) WresArgs& w = L->w;
-        const PkInputWait wait = {p.ctl, &s_err, deadline, l, xcd};
+        const PkInputWait wait = {p.ctl, &s_err, deadline, l, xcd, target};
         for (uint32_t v = rank; v < (uint32_t)nvirt; v += kPkPerXcd) {
             const uint32_t slice = v / w.ngroups, group = v - slice * w.ngroups;
             switch (variant) {
@@ -1207,21 +1213,16 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
         // this workgroup's share of layer l is stored: count it in
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
-        if (threadIdx.x == 0)
-            __hip_atomic_fetch_add(&p.ctl->arrive[(xcd * kPkMaxLayers + l) * 16], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) {
+            const uint32_t found = __hip_atomic_fetch_add(&p.ctl->arrive[(xcd * kPkMaxLayers + l) * 16], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            target = (found & ~(uint32_t)(kPkPerXcd - 1)) + kPkPerXcd;
+        }
         __syncthreads();
     }
     if (threadIdx.x == 0 && s_err != 0) {
         atomicMax(&p.ctl->error, s_err);
         if (p.host_error != nullptr) atomicMax(p.host_error, s_err);
     }
-}
-
-// Zeroes a segment's counters ahead of its launch (a kernel rather than a memset node, so that a caller may capture the
-// list's launches into a graph).
-__global__ __launch_bounds__(256) void pk_clear_kernel(uint4* p, uint32_t n16) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
 }
 
 // ---- fixed workspace -----------------------------------------------------------------------------------------------------
@@ -1243,14 +1244,6 @@ int pk_variant_of(int tag) {
 }
 
 }  // namespace
-
-hipError_t pk_clear(void* p, uint32_t bytes, hipStream_t stream) {
-    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(p) % 16 != 0) return hipErrorInvalidValue;
-    const uint32_t n16 = bytes / 16;
-    if (n16 == 0) return hipSuccess;
-    hipLaunchKernelGGL(pk_clear_kernel, dim3((n16 + 255) / 256), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
-    return hipGetLastError();
-}
 
 hipError_t pk_workspace(int device, PkWorkspace* ws) {
     constexpr int kMaxDevices = 64;
