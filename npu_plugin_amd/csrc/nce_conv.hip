@@ -307,21 +307,24 @@ static int tiled_shape_for(const ConvArgs& a) {
     if (tls_launch.per_xcd) return 0;
     const int forced = options().tiled;
     if (forced >= 0) return forced;
-    // Measured over the ResNet-50 layer shapes at batch 32, 128 and 256 against the weights-resident kernels. The 128 x 128
-    // tile with steps of 128 bytes of the reduction (one barrier and one LDS round trip per 32 matrix instructions of a
-    // wave; input channels a multiple of 128) is 3-25 % ahead - 45 % for 3x3 over 512 channels - where the reduction is long
-    // and the output channels many: from 1024 bytes of reduction for 256 channels or more once there are ~200 workgroups
-    // (fewer leave CUs idle), for 128 channels from 384 workgroups; from 512 bytes only for grids of 384 workgroups or more
-    // and not for 256 channels over very many pixels, where the weights-resident kernels amortise their staging over many
-    // tiles per workgroup and win again. Shorter reductions and fewer channels always lose. The 64-byte-step shape (input
-    // channels not a multiple of 128) is 9 % slower and keeps the narrower window it was measured in.
+    // Fitted to a sweep of the ResNet-50 layer shapes at batch 32, 64, 128 and 256 (each layer alone, every kernel forced)
+    // and to the whole graph at those batches. The 128 x 128 tile with steps of 128 bytes of the reduction (one barrier and
+    // one LDS round trip per 32 matrix instructions of a wave; input channels a multiple of 128) is 3-25 % ahead of the
+    // weights-resident kernels - 45 % for 3x3 over 512 channels - where the reduction is long and the output channels are
+    // many. Inside the graph a launch of it costs ~1.5 us more than alone (the layer-alone sweep repeats one kernel, whose
+    // weights then stay in L2 and whose launches overlap their own tails), so grids whose gain alone is 1-2 us are left to
+    // the weights-resident kernels: from 1024 bytes of reduction it takes 384 workgroups (196 from 4096 bytes), from 512
+    // bytes 512 workgroups of at least 256 channels - but not 256..511 channels over more than 1024 workgroups, where the
+    // weights-resident kernels amortise their staging over many tiles per workgroup and win again. Shorter reductions and
+    // fewer than 128 channels always lose. The 64-byte-step shape (input channels not a multiple of 128) is 9 % slower and
+    // keeps the narrower window it was measured in.
     const int64_t k = (int64_t)a.KY * a.KX * a.IC;
     if (a.IC % 64 != 0 || a.dw != 0 || k < 512 || a.bc < 128) return 0;
     const int64_t groups = (((int64_t)a.M + 127) / 128) * ((a.bc + 127) / 128);
     if (a.IC % 128 != 0) return k >= 1024 && a.bc >= 256 && groups >= 384 && groups <= 1024 ? 1 : 0;
     bool use;
-    if (k >= 1024) use = a.bc >= 256 ? groups >= 200 : groups >= 384;
-    else use = a.bc >= 256 && groups >= 384 && (a.bc >= 512 || groups <= 1024);
+    if (k >= 1024) use = groups >= (k >= 4096 ? 196 : 384);
+    else use = a.bc >= 256 && groups >= 512 && (a.bc >= 512 || groups <= 1024);
     return use ? 5 : 0;
 }
 
