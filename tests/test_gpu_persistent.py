@@ -71,3 +71,75 @@ def test_persistent_wait_limit_reports_and_falls_back(tuned):
         got = dg.buffers[L.dst].cpu().numpy()
         assert np.array_equal(got, want[L.dst]), f"{L.name}: {(got != want[L.dst]).sum()} bytes differ"
     dg.task_list.destroy()
+
+
+def _arena_buffers(graph, device="cuda:0"):
+    """The graph's activation tensors placed in ONE arena the way a memory planner would: a tensor's bytes are free again
+    after its last reader, and later tensors - of other shapes, hence other batch strides - take them (first fit, 256-byte
+    granules). Layers of a persistent segment run ahead of each other per XCD, so such reuse inside a segment would corrupt
+    data: the segment builder has to see the overlap and cut the segment there."""
+    import torch
+    last_use = {}
+    for j, L in enumerate(graph.layers):
+        for t in (L.src, L.src2, L.dst):
+            if t >= 0:
+                last_use[t] = j
+    last_use[graph.output] = len(graph.layers)
+    born = {0: -1}
+    for j, L in enumerate(graph.layers):
+        born[L.dst] = j
+    size = {t: (int(np.prod(s)) + 255) // 256 * 256 for t, s in enumerate(graph.tensors)}
+    placed = {}      # tensor -> (offset, size)
+    order = sorted(born, key=lambda t: born[t])
+    total = 0
+    for t in order:
+        live = [(o, s) for u, (o, s) in placed.items() if last_use[u] >= born[t]]   # (a layer's inputs outlive its output's birth)
+        live.sort()
+        off = 0
+        for o, s in live:
+            if off + size[t] <= o:
+                break
+            off = max(off, o + s)
+        placed[t] = (off, size[t])
+        total = max(total, off + size[t])
+    arena = torch.zeros(total, dtype=torch.uint8, device=device)
+    bufs = []
+    for t, shape in enumerate(graph.tensors):
+        off, _ = placed[t]
+        bufs.append(arena[off:off + int(np.prod(shape))].view(*shape))
+    shared = sum(s for _, s in placed.values()) - total
+    return arena, bufs, shared
+
+
+@pytest.mark.parametrize("no_alloc", [False, True])
+def test_persistent_with_reused_activation_memory(tuned, no_alloc):
+    """Activations in a planner-style arena (tensors reuse each other's bytes): persistent segments must stop where two
+    layers would touch the same bytes in different batch shares. The network output must equal the oracle's."""
+    import torch
+    from npu_plugin_amd import workloads as W
+    executor = _executor(NCE_HIP_PERSISTENT="1")
+    graph = K.ResNet50Graph(batch=16, size=64)
+    x = graph.make_input()
+    print(f"[case] resnet50 graph in an arena, persistent, no_alloc={no_alloc}", flush=True)
+    want = K.run_graph_oracle(graph, x)
+    arena, bufs, shared = _arena_buffers(graph)
+    assert shared > 0, "the arena does not reuse any memory"
+    bufs[0].copy_(torch.from_numpy(x))
+    weights = [torch.from_numpy(L.weights).to("cuda:0") if L.weights is not None else None for L in graph.layers]
+    tables = [torch.from_numpy(L.table).to("cuda:0") if L.table is not None else None for L in graph.layers]
+    tasks = graph.build_tasks(bufs, weights, tables)
+    tl = executor.task_list()
+    for t in tasks:
+        tl.append(t)
+    stream = torch.cuda.current_stream().cuda_stream
+    for rep in range(3):
+        bufs[0].copy_(torch.from_numpy(x))  # (the input's bytes may have been reused too)
+        torch.cuda.synchronize()
+        (tl.enqueue_no_alloc if no_alloc else tl.enqueue)(stream)
+        executor.synchronize(stream)
+        got = bufs[graph.output].cpu().numpy()
+        assert np.array_equal(got, want[graph.output]), f"run {rep}: {(got != want[graph.output]).sum()} bytes of the output differ"
+    text = executor.log()
+    print(text[-800:], flush=True)
+    assert "persistent launch" in text, "no persistent segment was formed"
+    tl.destroy()
