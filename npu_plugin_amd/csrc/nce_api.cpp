@@ -517,18 +517,18 @@ PkAlt pk_alternate(const Plan& p, const Plan* q) {
     TaskDev pd = p.dev;
     pd.in.n = pd.out.n = n / 8;
     std::vector<nce::RecordedLaunch> rec;
-    const nce::LaunchContext saved = nce::tls_launch;
-    nce::tls_launch.record = &rec;
-    nce::tls_launch.per_xcd = true;
     hipError_t e;
-    if (q != nullptr) {
-        TaskDev qd = q->dev;
-        qd.in.n = qd.in2.n = qd.out.n = n / 8;
-        e = nce::launch_conv_fused_add(pd, p.boxes[0], qd, q->boxes[0], nullptr);
-    } else {
-        e = nce::launch_conv(pd, p.boxes[0], nullptr);
+    {
+        const ScopedLaunch ctx(nce::tls_launch.opt, &rec);  // (restores the caller's recorder, also when a launch throws)
+        nce::tls_launch.per_xcd = true;
+        if (q != nullptr) {
+            TaskDev qd = q->dev;
+            qd.in.n = qd.in2.n = qd.out.n = n / 8;
+            e = nce::launch_conv_fused_add(pd, p.boxes[0], qd, q->boxes[0], nullptr);
+        } else {
+            e = nce::launch_conv(pd, p.boxes[0], nullptr);
+        }
     }
-    nce::tls_launch = saved;
     if (e != hipSuccess || rec.size() != 1 || !nce::wres_pk_has_variant(rec[0].tag)) return alt;
     alt.launch = std::move(rec[0]);
     alt.d_in = (int64_t)(n / 8) * p.dev.in.sn;
