@@ -393,6 +393,26 @@ def main():
             others["cfg3_chain"] = measure_chain(ex, args.steps, args.warmup)
         if args.workload != "cfg5":
             others["cfg5"] = measure_graph(ex, graph_steps, graph_warm)
+        # The same graph with the opt-in persistent segments (an executor created under NCE_HIP_PERSISTENT=1): runs of
+        # weights-resident convolutions as one launch each. Not the headline: the default path is.
+        saved = os.environ.get("NCE_HIP_PERSISTENT")
+        os.environ["NCE_HIP_PERSISTENT"] = "1"
+        try:
+            ex_pk = nce.Executor(device_id=0, log_level=1)
+            try:
+                r = measure_graph(ex_pk, graph_steps, graph_warm)
+                ex_pk.synchronize(torch.cuda.current_stream().cuda_stream)  # (reports a persistent launch that gave up)
+                r["roofline"]["note"] = "NCE_HIP_PERSISTENT=1: launches 12..53 of the graph as one persistent launch"
+                others["cfg5_persistent_segments"] = r
+            finally:
+                ex_pk.destroy()
+        except Exception as e:  # the headline does not depend on this line
+            others["cfg5_persistent_segments"] = {"error": str(e)[:200]}
+        finally:
+            if saved is None:
+                del os.environ["NCE_HIP_PERSISTENT"]
+            else:
+                os.environ["NCE_HIP_PERSISTENT"] = saved
         line["other_workloads"] = others
         if not args.no_scaled:
             scaled = {}
