@@ -592,10 +592,7 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, boo
     nce_executor_s* const ex = list->ex;
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ex->device) != hipSuccess || cus != nce::kPkWorkgroups) return NCE_RESULT_SUCCESS;
-    if (!fixed_ws && ex->pk_host_error == nullptr) {
-        if (hipHostMalloc(reinterpret_cast<void**>(&ex->pk_host_error), 64, hipHostMallocDefault) != hipSuccess) return NCE_RESULT_SUCCESS;
-        *ex->pk_host_error = 0;
-    }
+    if (!fixed_ws && ex->pk_host_error == nullptr) return NCE_RESULT_SUCCESS;  // (no error word: no persistent launches)
     std::vector<nce::RecordedLaunch> out;
     size_t i = 0;
     const size_t n = list->launches.size();
@@ -712,6 +709,12 @@ nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* 
         }
         // The fixed workspace's address on this device (nceTaskListEnqueueNoAlloc); everything else works without it.
         if (hipSetDevice(desc.device_id) == hipSuccess) {
+            // (persistent launches report through a pinned host word; made here, once, rather than by the first list that
+            // needs it - lists of one executor may be prepared from several threads)
+            if (ex->opt.persistent != 0 && hipHostMalloc(reinterpret_cast<void**>(&ex->pk_host_error), 64, hipHostMallocDefault) == hipSuccess)
+                *ex->pk_host_error = 0;
+            else
+                ex->pk_host_error = nullptr;
             const hipError_t we = nce::pk_workspace(desc.device_id, &ex->ws);
             ex->ws_ok = we == hipSuccess;
             if (!ex->ws_ok) lg->add(2, "fixed workspace not available on device %d: %s", desc.device_id, hipGetErrorString(we));
