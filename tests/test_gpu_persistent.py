@@ -26,7 +26,7 @@ def _executor(**env):
 
 
 @pytest.mark.parametrize("batch,size", [(8, 64), (16, 96)])
-def test_resnet50_graph_persistent(tuned, batch, size):
+def test_resnet50_graph_persistent(batch, size):
     import torch
     executor = _executor(NCE_HIP_PERSISTENT="1")
     graph = K.ResNet50Graph(batch=batch, size=size)
@@ -48,7 +48,7 @@ def test_resnet50_graph_persistent(tuned, batch, size):
     dg.task_list.destroy()
 
 
-def test_persistent_wait_limit_reports_and_falls_back(tuned):
+def test_persistent_wait_limit_reports_and_falls_back():
     """A wait limit of zero makes the segment's first unsatisfied wait give up (every workgroup still leaves the kernel
     normally): the synchronise call must report the failure, and the next enqueue - persistent launches now off for
     the executor - must produce the oracle's tensors through ordinary launches."""
@@ -112,11 +112,10 @@ def _arena_buffers(graph, device="cuda:0"):
 
 
 @pytest.mark.parametrize("no_alloc", [False, True])
-def test_persistent_with_reused_activation_memory(tuned, no_alloc):
+def test_persistent_with_reused_activation_memory(no_alloc):
     """Activations in a planner-style arena (tensors reuse each other's bytes): persistent segments must stop where two
     layers would touch the same bytes in different batch shares. The network output must equal the oracle's."""
     import torch
-    from npu_plugin_amd import workloads as W
     executor = _executor(NCE_HIP_PERSISTENT="1")
     graph = K.ResNet50Graph(batch=16, size=64)
     x = graph.make_input()

@@ -30,7 +30,7 @@ def _tensors(dg, graph):
     return {L.dst: dg.buffers[L.dst].cpu().numpy() for L in graph.layers}
 
 
-def test_no_alloc_enqueue_matches_enqueue(tuned):
+def test_no_alloc_enqueue_matches_enqueue():
     import torch
     stream = torch.cuda.current_stream().cuda_stream
     ex_ref = _executor(NCE_HIP_PERSISTENT="1")
@@ -73,7 +73,7 @@ def test_no_alloc_enqueue_matches_enqueue(tuned):
         dg.task_list.destroy()
 
 
-def test_no_alloc_enqueue_rejects_more_layers_than_the_workspace_holds(tuned):
+def test_no_alloc_enqueue_rejects_more_layers_than_the_workspace_holds():
     import torch
     import npu_plugin_amd as nce
     stream = torch.cuda.current_stream().cuda_stream
