@@ -189,7 +189,8 @@ nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream);
  * does for an executor created under NCE_HIP_PERSISTENT=1 - runs of consecutive weights-resident convolutions as one
  * persistent launch each - but keeps those launches' layer tables, counters and error word in a fixed array in device
  * memory that belongs to the library (281 KiB per GPU, held until the process ends) instead of allocating them, and
- * calls neither hipMalloc nor hipFree. Limits: the persistent launches of one list may cover at most 64 layers together
+ * calls neither hipMalloc nor hipFree. (The tables travel to that array through 248 KiB of pinned host memory that every
+ * executor with a device gets when it is created.) Limits: the persistent launches of one list may cover at most 64 layers together
  * (more: NCE_RESULT_ERROR_UNSUPPORTED, nothing is launched); a list that nceTaskListEnqueue has prepared with device
  * allocations is refused (NCE_RESULT_ERROR_INVALID_ARGUMENT). Every call on a GPU shares that GPU's array: calls whose
  * launches may overlap on the GPU (two streams, two executors, two processes do not share it) race and must be

@@ -27,8 +27,16 @@ struct nce_executor_s {
     nce::PkWorkspace ws;
     bool ws_ok = false;
     std::atomic<bool> ws_used{false};   // a launch that reports through ws.error may be in flight
+    // Pinned staging for the layer tables on their way into the workspace (made at creation, so that the enqueue itself
+    // neither allocates nor leaves the runtime to pin pageable memory), and the event that says the last copy has left it.
+    std::mutex ws_mu;
+    uint8_t* ws_staging = nullptr;
+    hipEvent_t ws_event = nullptr;
+    bool ws_event_pending = false;
     ~nce_executor_s() {
         if (pk_host_error != nullptr) (void)hipHostFree(pk_host_error);
+        if (ws_staging != nullptr) (void)hipHostFree(ws_staging);
+        if (ws_event != nullptr) (void)hipEventDestroy(ws_event);
     }
 };
 
@@ -715,7 +723,9 @@ nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* 
                 *ex->pk_host_error = 0;
             else
                 ex->pk_host_error = nullptr;
-            const hipError_t we = nce::pk_workspace(desc.device_id, &ex->ws);
+            hipError_t we = nce::pk_workspace(desc.device_id, &ex->ws);
+            if (we == hipSuccess) we = hipHostMalloc(reinterpret_cast<void**>(&ex->ws_staging), ex->ws.table_bytes, hipHostMallocDefault);
+            if (we == hipSuccess) we = hipEventCreateWithFlags(&ex->ws_event, hipEventDisableTiming);
             ex->ws_ok = we == hipSuccess;
             if (!ex->ws_ok) lg->add(2, "fixed workspace not available on device %d: %s", desc.device_id, hipGetErrorString(we));
         }
@@ -840,8 +850,18 @@ nce_result_t enqueue_list(nce_task_list_handle_t list, void* hip_stream, bool fi
             list->prepared = true;
         }
         if (list->fixed_ws && list->has_segments) {
-            // The workspace holds whatever the last list to use it left there: this list's tables go in ahead of its launches.
-            const hipError_t e = hipMemcpyAsync(ex->ws.table, list->ws_table.data(), list->ws_table.size(), hipMemcpyHostToDevice, stream);
+            // The workspace holds whatever the last list to use it left there: this list's tables go in ahead of its launches,
+            // through the executor's pinned staging buffer (once the previous copy out of it has finished).
+            std::lock_guard<std::mutex> ws_lock(ex->ws_mu);
+            hipError_t e = ex->ws_event_pending ? hipEventSynchronize(ex->ws_event) : hipSuccess;
+            if (e == hipSuccess) {
+                memcpy(ex->ws_staging, list->ws_table.data(), list->ws_table.size());
+                e = hipMemcpyAsync(ex->ws.table, ex->ws_staging, list->ws_table.size(), hipMemcpyHostToDevice, stream);
+            }
+            if (e == hipSuccess) {
+                e = hipEventRecord(ex->ws_event, stream);
+                ex->ws_event_pending = e == hipSuccess;
+            }
             if (e != hipSuccess) {
                 ex->log->add(1, "copy of the layer tables to the fixed workspace failed: %s", hipGetErrorString(e));
                 return NCE_RESULT_ERROR_UNKNOWN;
