@@ -126,7 +126,10 @@ typedef struct nce_ppe_task_t {
 } nce_ppe_task_t;
 
 /* Bits of nce_cluster_task_desc_t::flags = the boolean attributes of NCEClusterTask
- * (ops.td:2803-2817). None of them is implemented: any set bit -> NCE_RESULT_ERROR_UNSUPPORTED. */
+ * (ops.td:2803-2817). NCE_FLAG_IS_INPLACE is accepted on ELTWISE tasks whose output IS one of the two inputs (the same
+ * address, strides and storage type: what convert_eltwise_to_in_place.cpp:114-200 produces); on any other task or with
+ * any other output it is NCE_RESULT_ERROR_INVALID_ARGUMENT. The other attributes are not implemented: a set bit ->
+ * NCE_RESULT_ERROR_UNSUPPORTED. */
 #define NCE_FLAG_IS_CONTINUED (1u << 0)
 #define NCE_FLAG_IS_SEGMENTED (1u << 1)
 #define NCE_FLAG_INPUT_CHANNELS_COMPRESSION (1u << 2)

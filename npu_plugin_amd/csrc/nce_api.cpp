@@ -355,7 +355,12 @@ nce_result_t build_boxes(nce_log_s* log, const nce_cluster_task_desc_t* t, const
 
 nce_result_t make_plan(nce_log_s* log, const nce_cluster_task_desc_t* t, Plan* plan) {
     if (t == nullptr) FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "task descriptor is null");
-    if (t->flags != 0) FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "task flags 0x%x: continued / segmented / compressed / superdense / in-place / permute-quantize / small-kernel tasks are not supported", t->flags);
+    // is_inplace is the one boolean attribute with a meaning here (below, with the ELTWISE checks); the others change what the
+    // hardware computes or how operands are stored.
+    if ((t->flags & ~NCE_FLAG_IS_INPLACE) != 0)
+        FAIL(NCE_RESULT_ERROR_UNSUPPORTED, "task flags 0x%x: continued / segmented / compressed / superdense / permute-quantize / small-kernel tasks are not supported", t->flags & ~NCE_FLAG_IS_INPLACE);
+    if ((t->flags & NCE_FLAG_IS_INPLACE) != 0 && t->task_type != NCE_TASK_ELTWISE)
+        FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "is_inplace is an attribute of ELTWISE tasks");
     TaskDev& d = plan->dev;
     memset(&d, 0, sizeof(d));
     plan->task_type = t->task_type;
@@ -389,6 +394,16 @@ nce_result_t make_plan(nce_log_s* log, const nce_cluster_task_desc_t* t, Plan* p
         if (d.in2.is_signed != d.in.is_signed)
             FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "ELTWISE inputs must share the storage type");  // eltwise_utils.cpp:15-65
         d.ky = d.kx = d.sy = d.sx = 1;
+        if ((t->flags & NCE_FLAG_IS_INPLACE) != 0) {
+            // The reference replaces an in-place eltwise's output buffer by one of its input buffers, which must have the
+            // output's element type and allocation size (convert_eltwise_to_in_place.cpp:114-200): the output must BE one of
+            // the inputs. Every output element depends on the same element of the inputs only, so the kernels need nothing else.
+            const auto same = [](const nce::TensorDev& x, const nce::TensorDev& y) {
+                return x.data == y.data && x.sn == y.sn && x.sh == y.sh && x.sw == y.sw && x.sc == y.sc && x.is_signed == y.is_signed;
+            };
+            if (!same(d.out, d.in) && !same(d.out, d.in2))
+                FAIL(NCE_RESULT_ERROR_INVALID_ARGUMENT, "is_inplace: the output must be one of the two inputs (same address, strides and storage type)");
+        }
     } else {
         if ((r = check_kernel(log, t)) != NCE_RESULT_SUCCESS) return r;
         if ((r = check_out_shape(log, t, d.in, d.out)) != NCE_RESULT_SUCCESS) return r;

@@ -176,6 +176,30 @@ def test_eltwise_variants(executor, kw):
 
 # ---- variants: any tiling of the output box gives the same bytes ---------------------------------
 
+@pytest.mark.parametrize("onto", [1, 2])
+@pytest.mark.parametrize("variants", [False, True])
+def test_eltwise_in_place(executor, onto, variants):
+    """An eltwise flagged is_inplace writes its output over its first (second) input; the bytes are those of the same
+    add into a separate tensor."""
+    import torch
+    case = K.eltwise_case(91, 2, 9, 13, 48, signed=True, zp_a=-3, zp_b=12, out_zp=-100) if onto == 2 else K.eltwise_case(91, 2, 9, 13, 48)
+    if variants:
+        case.variants = [((0, 0, 0), (12, 3, 47)), ((0, 4, 0), (12, 8, 15)), ((0, 4, 16), (12, 8, 47))]
+    print(f"[case] eltwise in place onto input {onto}, variants={variants}", flush=True)
+    want = K.run_oracle(case)
+    a = torch.from_numpy(case.input).to("cuda:0")
+    b = torch.from_numpy(case.weights).to("cuda:0")
+    out = a if onto == 1 else b
+    task = K.build_task(case, a, b, None, out)
+    task.desc.flags = 1 << 4
+    stream = torch.cuda.current_stream().cuda_stream
+    executor.enqueue(task, stream)
+    executor.synchronize(stream)
+    assert np.array_equal(out.cpu().numpy(), want)
+    other = b if onto == 1 else a
+    assert np.array_equal(other.cpu().numpy(), case.weights if onto == 1 else case.input), "the other input was touched"
+
+
 def _tilings(oh, ow, oc):
     yield [((0, 0, 0), (ow - 1, oh // 2 - 1, oc - 1)), ((0, oh // 2, 0), (ow - 1, oh - 1, oc - 1))]       # split over height
     yield [((0, 0, 0), (ow - 1, oh - 1, 15)), ((0, 0, 16), (ow - 1, oh - 1, oc - 1))]                     # split over channels

@@ -36,6 +36,27 @@ def test_null_and_flags(validator):
     assert rc == abi.ERROR_UNSUPPORTED and "superdense" in log
 
 
+def test_is_inplace_only_for_an_eltwise_whose_output_is_an_input(validator):
+    """is_inplace (bit 4): the reference rewrites such an eltwise to write one of its input buffers
+    (src/vpux_compiler/src/dialect/VPUIP/passes/convert_eltwise_to_in_place.cpp:114-200)."""
+    conv = task_of(K.cfg1())
+    conv.desc.flags = 1 << 4
+    rc, log = code(validator, conv)
+    assert rc == abi.ERROR_INVALID_ARGUMENT and "ELTWISE" in log
+    c = K.cfg4(n=1)
+    apart = task_of(c)
+    apart.desc.flags = 1 << 4
+    rc, log = code(validator, apart)
+    assert rc == abi.ERROR_INVALID_ARGUMENT and "one of the two inputs" in log
+    for alias in (c.input, c.weights):  # the output is the first / the second input
+        t = task_of(c, out=alias)
+        t.desc.flags = 1 << 4
+        assert code(validator, t)[0] == abi.SUCCESS
+    both = task_of(c, out=c.input)
+    both.desc.flags = (1 << 4) | (1 << 3)
+    assert code(validator, both)[0] == abi.ERROR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("task_type", [4, 6, 7, 99])  # FCL, IDENTITY, CMCONV, garbage
 def test_unsupported_task_types(validator, task_type):
     t = task_of(K.cfg1())
