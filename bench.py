@@ -109,6 +109,28 @@ def make_scaled_workloads():
     }
 
 
+MIN_WARM_S = 0.03  # every measurement is preceded by at least this much GPU work (clocks ramp on an idle device)
+
+
+STEPS_RUN = [0]  # steps of the main workload enqueued so far, warm-up included (what --marks reports)
+
+
+def warm_up(run, count, per_run=1):
+    """Runs `run()` at least `count` times and for at least MIN_WARM_S of wall time, then waits for the device: the
+    timed region that follows sees a device at its working clocks whatever step count the caller chose."""
+    import torch
+    t0 = time.perf_counter()
+    done = 0
+    while done < max(1, count) or time.perf_counter() - t0 < MIN_WARM_S:
+        run()
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()  # (keeps the wall clock honest: enqueues run ahead of the device)
+    torch.cuda.synchronize()
+    STEPS_RUN[0] += done * per_run
+    return done
+
+
 def time_task(ex, dc, steps, warmup):
     """Returns (wall seconds per step, event seconds per step)."""
     import torch
@@ -119,8 +141,7 @@ def time_task(ex, dc, steps, warmup):
     timed = ex.task_list()
     for _ in range(steps):
         timed.append(dc.task)
-    warm.enqueue(stream)
-    torch.cuda.synchronize()
+    warm_up(lambda: warm.enqueue(stream), 1, per_run=max(warmup, 1))
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -165,8 +186,7 @@ def per_layer_table(ex, dg, reps=10):
         tl = ex.task_list()
         for _ in range(reps):
             tl.append(task)
-        tl.enqueue(stream)
-        torch.cuda.synchronize()
+        warm_up(lambda: tl.enqueue(stream), 1)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         tl.enqueue(stream)
@@ -189,9 +209,7 @@ def measure_graph(ex, steps, warmup, batch=32, per_layer=False):
     graph = W.ResNet50Graph(batch=batch)
     dg = W.DeviceGraph(graph, ex, graph.make_input())
     stream = torch.cuda.current_stream().cuda_stream
-    for _ in range(max(1, warmup)):
-        dg.run(stream)
-    torch.cuda.synchronize()
+    warm_up(lambda: dg.run(stream), warmup)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
@@ -278,8 +296,7 @@ def measure_chain(ex, steps, warmup):
         for _ in range(k):
             for t in tasks:
                 tl.append(t)
-    warm.enqueue(stream)
-    torch.cuda.synchronize()
+    warm_up(lambda: warm.enqueue(stream), 1, per_run=max(warmup, 1))
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
@@ -341,6 +358,9 @@ def main():
         del src, dst
 
     graph_steps, graph_warm = args.steps, max(1, args.warmup)
+    # The side workloads are 3-15 us per step: they are timed over at least 200 steps whatever --steps says, so that their
+    # figures do not depend on the step count chosen for the headline.
+    side_steps = max(args.steps, 200)
     if args.workload == "cfg5":
         case, bound = None, "mfma"
         main_res = measure_graph(ex, graph_steps, graph_warm, per_layer=args.per_layer)
@@ -377,20 +397,15 @@ def main():
         "config": {"workload": workload_name, "ops_per_step": main_res["ops_per_step"], "bytes_per_step": main_res["bytes_per_step"]},
         "roofline": main_res["roofline"],
     }
-    if not args.no_cpu:
-        if case is not None:
-            line["cpu_baseline"] = cpu_baseline(case, bound)
-        elif args.workload == "cfg5":
-            line["cpu_baseline"] = cpu_baseline_graph()
     if not args.no_others:
         others = {}
         for name, (mk, bd) in workloads.items():
             if name == args.workload:
                 continue
-            _, r = measure(ex, name, mk, bd, args.steps, args.warmup)
+            _, r = measure(ex, name, mk, bd, side_steps, args.warmup)
             others[name] = r
         if args.workload != "cfg3_chain":
-            others["cfg3_chain"] = measure_chain(ex, args.steps, args.warmup)
+            others["cfg3_chain"] = measure_chain(ex, side_steps, args.warmup)
         if args.workload != "cfg5":
             others["cfg5"] = measure_graph(ex, graph_steps, graph_warm)
         # The same graph with the opt-in persistent segments (an executor created under NCE_HIP_PERSISTENT=1): runs of
@@ -421,6 +436,11 @@ def main():
                 scaled[name] = r
             line["scaled_workloads"] = scaled
     ex.destroy()
+    if not args.no_cpu:  # after every GPU measurement: seconds of host-only work would let the device clocks fall
+        if case is not None:
+            line["cpu_baseline"] = cpu_baseline(case, bound)
+        elif args.workload == "cfg5":
+            line["cpu_baseline"] = cpu_baseline_graph()
     print(json.dumps(line))
 
 

@@ -187,18 +187,22 @@ nce_result_t nceClusterTaskEnqueue(nce_executor_handle_t executor, const nce_clu
 nce_result_t nceTaskListCreate(nce_executor_handle_t executor, nce_task_list_handle_t* list);
 nce_result_t nceTaskListAppend(nce_task_list_handle_t list, const nce_cluster_task_desc_t* task);
 nce_result_t nceTaskListEnqueue(nce_task_list_handle_t list, void* hip_stream);
-/* nceTaskListEnqueue for callers that cannot allocate device memory (code under stream capture, tight serving loops,
- * harnesses that forbid hipMalloc). It has no counterpart in the reference. It runs the list the way nceTaskListEnqueue
- * does for an executor created under NCE_HIP_PERSISTENT=1 - runs of consecutive weights-resident convolutions as one
- * persistent launch each - but keeps those launches' layer tables, counters and error word in a fixed array in device
- * memory that belongs to the library (281 KiB per GPU, held until the process ends) instead of allocating them, and
- * calls neither hipMalloc nor hipFree. (The tables travel to that array through 248 KiB of pinned host memory that every
- * executor with a device gets when it is created.) Limits: the persistent launches of one list may cover at most 64 layers together
- * (more: NCE_RESULT_ERROR_UNSUPPORTED, nothing is launched); a list that nceTaskListEnqueue has prepared with device
- * allocations is refused (NCE_RESULT_ERROR_INVALID_ARGUMENT). Every call on a GPU shares that GPU's array: calls whose
- * launches may overlap on the GPU (two streams, two executors, two processes do not share it) race and must be
- * serialised by the caller. Failures of a persistent launch are reported by nceExecutorSynchronize, as for
- * nceTaskListEnqueue. */
+/* nceTaskListEnqueue for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. It runs the list the way nceTaskListEnqueue does for an executor
+ * created under NCE_HIP_PERSISTENT=1 - runs of consecutive weights-resident convolutions as one persistent launch each -
+ * but keeps those launches' layer tables, counters and error word in a fixed array in device memory that belongs to the
+ * library (281 KiB per GPU, held until the process ends) instead of allocating them, and calls neither hipMalloc nor
+ * hipFree. (The tables travel to that array through 248 KiB of pinned host memory that every executor with a device
+ * gets when it is created.) Limits: the array holds the tables of 64 layers per list - persistent launches beyond that
+ * run as the ordinary launches they were made from (which allocate nothing either); a list that nceTaskListEnqueue has
+ * prepared with device allocations is refused (NCE_RESULT_ERROR_INVALID_ARGUMENT); a stream that is being captured is
+ * refused (NCE_RESULT_ERROR_UNSUPPORTED: every call re-stages its tables through the executor's one pinned buffer and
+ * waits on an event, neither of which a graph replay would repeat - the call is eager only). Every call on a GPU shares
+ * that GPU's array: calls whose launches may overlap on the GPU (two streams, two executors; two processes do not
+ * share it) race and must be serialised by the caller. Failures of a persistent launch are reported by
+ * nceExecutorSynchronize, as for nceTaskListEnqueue; because the array's error word and counters are shared, a failure
+ * found by one executor of a GPU is reported by the next nceExecutorSynchronize of every other executor that used this
+ * entry point on that GPU as well. */
 nce_result_t nceTaskListEnqueueNoAlloc(nce_task_list_handle_t list, void* hip_stream);
 nce_result_t nceTaskListDestroy(nce_task_list_handle_t list);
 

@@ -27,6 +27,10 @@ struct nce_executor_s {
     nce::PkWorkspace ws;
     bool ws_ok = false;
     std::atomic<bool> ws_used{false};   // a launch that reports through ws.error may be in flight
+    // The workspace (error word, counters) is shared by every executor of the device: whichever executor reads a raised
+    // error word clears it, so the failure is also counted per device (ws_failures below) and every executor compares
+    // that count with the one it last saw.
+    uint32_t ws_failures_seen = 0;
     // Pinned staging for the layer tables on their way into the workspace (made at creation, so that the enqueue itself
     // neither allocates nor leaves the runtime to pin pageable memory), and the event that says the last copy has left it.
     std::mutex ws_mu;
@@ -41,6 +45,12 @@ struct nce_executor_s {
 };
 
 thread_local nce::LaunchContext nce::tls_launch;
+
+namespace {
+// Launches of the fixed workspace that gave up, per device and process (see nce_executor_s::ws_failures_seen).
+constexpr int kWsMaxDevices = 64;
+std::atomic<uint32_t> ws_failures[kWsMaxDevices];
+}  // namespace
 
 namespace {
 
@@ -645,9 +655,13 @@ nce_result_t build_segments(nce_task_list_s* list, std::vector<PkAlt>& alts, boo
         void* d_ctl = nullptr;
         if (fixed_ws && e == hipSuccess) {
             if (list->ws_table.size() + table.size() > ex->ws.table_bytes) {
-                ex->log->add(1, "task list: its persistent launches cover more than %d layers, the limit of the fixed workspace "
-                                "(nceTaskListEnqueueNoAlloc); use nceTaskListEnqueue or a shorter list", nce::kPkMaxLayers);
-                return NCE_RESULT_ERROR_UNSUPPORTED;
+                // The workspace holds the tables of kPkMaxLayers layers per list: what does not fit runs as the ordinary
+                // recorded launches it was made from (which allocate nothing either).
+                ex->log->add(2, "task list: launches %zu..%zu stay ordinary launches (the fixed workspace holds %d layers per list)",
+                             i, j - 1, nce::kPkMaxLayers);
+                for (size_t k = i; k < j; ++k) out.push_back(std::move(list->launches[k]));
+                i = j;
+                continue;
             }
             nce::PkArgs args;
             args.layers = ex->ws.table + list->ws_table.size();
@@ -741,7 +755,8 @@ nce_result_t nceExecutorCreate(nce_executor_desc_t desc, nce_executor_handle_t* 
             hipError_t we = nce::pk_workspace(desc.device_id, &ex->ws);
             if (we == hipSuccess) we = hipHostMalloc(reinterpret_cast<void**>(&ex->ws_staging), ex->ws.table_bytes, hipHostMallocDefault);
             if (we == hipSuccess) we = hipEventCreateWithFlags(&ex->ws_event, hipEventDisableTiming);
-            ex->ws_ok = we == hipSuccess;
+            ex->ws_ok = we == hipSuccess && desc.device_id < kWsMaxDevices;
+            if (ex->ws_ok) ex->ws_failures_seen = ws_failures[desc.device_id].load();
             if (!ex->ws_ok) lg->add(2, "fixed workspace not available on device %d: %s", desc.device_id, hipGetErrorString(we));
         }
     }
@@ -827,6 +842,16 @@ nce_result_t enqueue_list(nce_task_list_handle_t list, void* hip_stream, bool fi
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     try {
         std::lock_guard<std::mutex> lk(list->mu);
+        if (fixed_ws) {
+            // The form stages its layer tables through one pinned buffer and an event per executor: a captured copy would
+            // re-read, at every replay, whatever list staged last, and an event recorded while capturing cannot be waited
+            // for. So it is an eager-only entry point.
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+                ex->log->add(1, "nceTaskListEnqueueNoAlloc: the stream is being captured; this entry point cannot be recorded into a graph");
+                return NCE_RESULT_ERROR_UNSUPPORTED;
+            }
+        }
         if (fixed_ws && !ex->ws_ok) {
             ex->log->add(1, "nceTaskListEnqueueNoAlloc: the fixed workspace was not found on device %d when the executor was created", ex->device);
             return NCE_RESULT_ERROR_UNSUPPORTED;
@@ -935,6 +960,14 @@ nce_result_t nceExecutorSynchronize(nce_executor_handle_t executor, void* hip_st
             (void)hipMemset(executor->ws.error, 0, sizeof(ws_code));
             (void)hipMemset(executor->ws.ctl, 0, sizeof(nce::PkCtl));
             code = std::max(code, ws_code);
+            ws_failures[executor->device].fetch_add(1);
+        }
+        // (another executor of this device may have read and cleared the word first: its launches share the counters
+        // with ours, so a failure it found leaves this executor's outputs in doubt as well)
+        const uint32_t failures = ws_failures[executor->device].load();
+        if (failures != executor->ws_failures_seen) {
+            executor->ws_failures_seen = failures;
+            code = std::max<uint32_t>(code, 1);
         }
     }
     if (code != 0) {

@@ -1210,7 +1210,10 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
             }
             __syncthreads();  // every wave has left the LDS weights and tables
         }
-        // this workgroup's share of layer l is stored: count it in
+        // This workgroup's share of layer l is stored: count it in. Every wave first waits until the L2 has acknowledged
+        // all of its own stores (vmcnt(0), said explicitly: a workgroup-scope release need not wait for them), so that once
+        // the barrier below has passed, the whole workgroup's output is in the XCD's L2 before thread 0 arrives.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters untouched
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -1221,7 +1224,9 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
     }
     if (threadIdx.x == 0 && s_err != 0) {
         atomicMax(&p.ctl->error, s_err);
-        if (p.host_error != nullptr) atomicMax(p.host_error, s_err);
+        // (a plain store: any non-zero code reports the failure, and a read-modify-write on host memory needs atomic
+        // routing over the bus that a platform may lack)
+        if (p.host_error != nullptr) __hip_atomic_store(p.host_error, s_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
 
