@@ -71,9 +71,10 @@ struct Plan {
 // Sets the calling thread's launch context for the duration of one C-ABI call.
 struct ScopedLaunch {
     nce::LaunchContext saved;
-    ScopedLaunch(const nce::Options* opt, std::vector<nce::RecordedLaunch>* record) : saved(nce::tls_launch) {
+    ScopedLaunch(const nce::Options* opt, std::vector<nce::RecordedLaunch>* record, nce_log_s* log = nullptr) : saved(nce::tls_launch) {
         nce::tls_launch.opt = opt;
         nce::tls_launch.record = record;
+        nce::tls_launch.log = log;
     }
     ~ScopedLaunch() { nce::tls_launch = saved; }
 };
@@ -88,6 +89,17 @@ nce::Options read_options() {
         o.wres_forced = sscanf(e, "%d,%d,%d,%d", &o.wres[0], &o.wres[1], &o.wres[2], &o.wres[3]) == 4;
     if (const char* e = getenv("NCE_HIP_CONV_TILE")) o.halo_tile = atoi(e);
     if (const char* e = getenv("NCE_HIP_CONV_TILED")) o.tiled = atoi(e);
+    if (const char* e = getenv("NCE_HIP_CONV_PATCH")) {
+        int nf = 0, pr = 0;
+        const int got = sscanf(e, "%d,%d", &nf, &pr);
+        if (got == 2) {
+            o.patch = 1;
+            o.patch_nf = nf;
+            o.patch_pr = pr;
+        } else if (got == 1) {
+            o.patch = nf != 0 ? 1 : 0;
+        }
+    }
     o.no_fuse = getenv("NCE_HIP_NO_FUSE") != nullptr;
     if (const char* e = getenv("NCE_HIP_PERSISTENT")) o.persistent = atoi(e);
     if (const char* e = getenv("NCE_HIP_PERSISTENT_WAIT_US")) o.persistent_wait_us = std::max(0, atoi(e));
@@ -795,7 +807,7 @@ nce_result_t nceClusterTaskEnqueue(nce_executor_handle_t executor, const nce_clu
             return NCE_RESULT_ERROR_UNSUPPORTED;
         }
         if (hipSetDevice(executor->device) != hipSuccess) return NCE_RESULT_ERROR_UNKNOWN;
-        const ScopedLaunch ctx(&executor->opt, nullptr);
+        const ScopedLaunch ctx(&executor->opt, nullptr, executor->log);
         return launch_plan(executor, plan, static_cast<hipStream_t>(hip_stream));
     } catch (const std::bad_alloc&) {
         return NCE_RESULT_ERROR_OUT_OF_MEMORY;
@@ -871,7 +883,7 @@ nce_result_t enqueue_list(nce_task_list_handle_t list, void* hip_stream, bool fi
             const bool persistent = (fixed_ws || ex->opt.persistent != 0) && !ex->pk_off.load();
             std::vector<PkAlt> alts;
             {
-                const ScopedLaunch ctx(&ex->opt, &list->launches);
+                const ScopedLaunch ctx(&ex->opt, &list->launches, ex->log);
                 const nce_result_t r = run_plans(ex, list->plans, nullptr, persistent ? &alts : nullptr);
                 if (r != NCE_RESULT_SUCCESS) {
                     list->launches.clear();
@@ -879,7 +891,7 @@ nce_result_t enqueue_list(nce_task_list_handle_t list, void* hip_stream, bool fi
                 }
             }
             if (persistent) {
-                const ScopedLaunch ctx(&ex->opt, nullptr);
+                const ScopedLaunch ctx(&ex->opt, nullptr, ex->log);
                 const nce_result_t r = build_segments(list, alts, fixed_ws);
                 if (r != NCE_RESULT_SUCCESS) {
                     list->drop_prepared();

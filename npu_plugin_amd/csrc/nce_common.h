@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/nce_hip.h"
+#include "nce_log.h"
 
 namespace nce {
 
@@ -123,6 +124,8 @@ struct Options {
     int persistent = 0;       // NCE_HIP_PERSISTENT: task lists run runs of weights-resident convolutions as one persistent launch
     int persistent_wait_us = 2000000;  // NCE_HIP_PERSISTENT_WAIT_US: time after which a persistent launch's waits give up
     int tiled = -1;           // NCE_HIP_CONV_TILED: -1 automatic, 0 never, 1.. force that shape of the LDS-tiled kernel
+    int patch = -1;           // NCE_HIP_CONV_PATCH: -1 automatic, 0 never, 1 = wherever its conditions hold; "nf,pr" also forces its shape
+    int patch_nf = 0, patch_pr = 0;
     bool env_path = false;    // NCE_HIP_CONV_PATH was given at all (switches the conv + add fusion off, as NO_FUSE does)
 };
 
@@ -141,6 +144,7 @@ struct RecordedLaunch {
 struct LaunchContext {
     const Options* opt = nullptr;
     std::vector<RecordedLaunch>* record = nullptr;
+    nce_log_s* log = nullptr;   // the executor's log (kernel choices are noted there at level 3)
     // Per-XCD form: the task is one eighth of the batch, to be run by the 32 CUs of one XCD inside a persistent segment
     // (grids are sized for 32 CUs; only the weights-resident convolution kernels take part).
     bool per_xcd = false;

@@ -328,6 +328,14 @@ static int tiled_shape_for(const ConvArgs& a) {
     return use ? 5 : 0;
 }
 
+// Which convolutions take the patch kernel (both operands in LDS, every input byte fetched once per workgroup).
+static bool patch_wanted(const ConvArgs& a) {
+    if (tls_launch.per_xcd) return false;
+    const int forced = options().patch;
+    if (forced >= 0) return forced != 0;
+    return false;
+}
+
 hipError_t launch_conv_fused_add(const TaskDev& conv, const Box& cb, const TaskDev& add, const Box& ab, hipStream_t stream) {
     if (options().no_fuse || (options().env_path && !tls_launch.per_xcd)) return hipErrorNotSupported;
     const TensorDev& o = conv.out;
@@ -377,6 +385,8 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     // 3x3 over 1024 channels), the chunked weights-resident kernel for everything else and for what the halo
     // kernel rejects.
     hipError_t e = hipErrorNotSupported;
+    if (path == 0 && patch_wanted(a)) e = launch_conv_patch(a, stream, options().patch_nf, options().patch_pr);
+    if (e != hipErrorNotSupported) return e;
     if (const int shape = path == 0 ? tiled_shape_for(a) : 0) e = launch_conv_tiled(a, stream, shape);
     if (e != hipErrorNotSupported) return e;
     e = path == 0 ? launch_conv_wres(a, stream, a.KX != 3) : hipErrorNotSupported;

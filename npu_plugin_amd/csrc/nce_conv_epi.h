@@ -71,6 +71,23 @@ __device__ __forceinline__ void wres_epilogue(const CA& a, const EpiSmem& s, con
                                               const EpiPack& ep, FZP fz = nullptr, const uint4* other = nullptr) {
     const int ch0 = 4 * NF * q;
     if (ch0 >= noc) return;
+    if constexpr (PMODE == PPE_MODE_INT && BF > 1) {
+        // The 64-bit integer form runs one pixel fragment at a time: over all BF at once it needs more registers than the
+        // reduction loops of its callers, and then the whole kernel spills (a reload from scratch memory is a vector
+        // memory operation: the wait for it also waits for every activation load the kernel keeps in flight).
+#pragma unroll
+        for (int x = 0; x < BF; ++x) {
+            v4i a1[NF][1];
+#pragma unroll
+            for (int f = 0; f < NF; ++f) a1[f][0] = acc[f][x];
+            uint8_t* const d1[1] = {dst[x]};
+            const bool v1[1] = {valid[x]};
+            const int32_t w1[1] = {dws[x]};
+            wres_epilogue<NF, 1, PPE_MODE_INT, FZ>(a, s, sBfull, sCorr, a1, w1, q, noc, d1, v1, pu, ep, fz, FZ ? other + x : other);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+    }
     const PpeDev ppe_args = generic_copy<PpeDev>(a.ppe);
     static_assert(!FZ || NF == 4, "fused add: a lane holds 16 channels");
     uint32_t wo[BF][NF];

@@ -1,0 +1,37 @@
+// Pieces shared by the convolution kernels that keep matrix operands in LDS as 1 KiB blocks of 16 rows x 64 bytes filled
+// by global_load_lds_dwordx4 (16 bytes per lane from global memory straight into LDS) and read back as MFMA operands with
+// ds_read_b128: the bank-conflict-free placement of a row's four 16-byte pieces, and the wait-count immediate.
+#pragma once
+
+#include <stdint.h>
+
+namespace nce {
+namespace lds_detail {
+
+// How ds_read_b128 is served on gfx950 (measured with two lanes at a time reading one bank group at different addresses
+// while every other lane reads one common address): four clocks of sixteen lanes each, and the sixteen are not
+// neighbours - lanes {0-3, 12-15, 20-27}, then {4-11, 16-19, 28-31}, then the same two sets 32 higher. Within a set, lanes
+// that read different addresses of the same 16-byte bank group (64 banks x 4 bytes = sixteen groups, address / 16 mod 16)
+// take one more clock per extra address; every pattern timed fits that model (256 bytes/clock when the sixteen lanes of
+// each set cover the sixteen groups, 128 bytes/clock for a row-per-lane pattern without the right swizzle).
+//
+// In the operand read of v_mfma_i32_16x16x64_i8, lane 16 q + r takes piece q (16 bytes) of row r, so a set holds every
+// row exactly once: rows 0-3 and 12-15 with one piece, rows 4-11 with its neighbour q ^ 1.
+
+// Block of 16 rows x 64 bytes: piece p of row r sits at r * 64 + ((p ^ swz(r)) << 4). Rows r, r + 4, r + 8, r + 12 share
+// the bank groups 4 (r % 4) .. 4 (r % 4) + 3; with swz = 0, 3, 2, 1 for the four quarters of the rows, the pieces one set
+// takes from them (q, q ^ 1, q ^ 1, q) land at four different positions.
+__device__ __forceinline__ int swz(int r) {
+    return (-(r >> 2)) & 3;
+}
+
+// s_waitcnt immediate that waits until at most n vector-memory operations are outstanding (nothing else).
+constexpr int vmcnt_imm(int n) {
+    return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14);
+}
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+}  // namespace lds_detail
+}  // namespace nce

@@ -37,10 +37,10 @@ def tuned(monkeypatch):
     import npu_plugin_amd as nce
     made = []
 
-    def make(**env):
+    def make(log_level=2, **env):
         for k, v in env.items():
             monkeypatch.setenv(k, str(v))
-        ex = nce.Executor(device_id=0, log_level=2)
+        ex = nce.Executor(device_id=0, log_level=log_level)
         for k in env:
             monkeypatch.delenv(k)
         made.append(ex)
