@@ -333,6 +333,14 @@ static bool patch_wanted(const ConvArgs& a) {
     if (tls_launch.per_xcd) return false;
     const int forced = options().patch;
     if (forced >= 0) return forced != 0;
+    // Measured against the weights-resident kernels over the ResNet-50 shapes at batch 32 .. 256 (each layer alone): ahead
+    // by 6-17 % for 3x3 kernels at stride 1 over 64 input channels from about 100,000 output pixels and over 128 input
+    // channels from about 50,000 (64 output channels per slice, sixteen waves); level or behind for everything else - 1x1
+    // kernels (nothing to reuse), 256 and more input channels (a slice of 32 channels reads 0.75 KiB of LDS per matrix
+    // instruction) and small layers (too few patches for the CUs).
+    if (a.KY * a.KX < 2 || a.SY != 1 || a.SX != 1 || a.dw != 0 || a.bc < 64) return false;
+    if (a.IC == 64) return a.M >= 100000;
+    if (a.IC == 128) return a.M >= 50000;
     return false;
 }
 
@@ -385,7 +393,8 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     // 3x3 over 1024 channels), the chunked weights-resident kernel for everything else and for what the halo
     // kernel rejects.
     hipError_t e = hipErrorNotSupported;
-    if (path == 0 && patch_wanted(a)) e = launch_conv_patch(a, stream, options().patch_nf, options().patch_pr);
+    if (path == 0 && patch_wanted(a))
+        e = launch_conv_patch(a, stream, options().patch >= 0 ? options().patch_nf : 4, options().patch_pr, options().patch >= 0 ? options().patch_waves : 16);
     if (e != hipErrorNotSupported) return e;
     if (const int shape = path == 0 ? tiled_shape_for(a) : 0) e = launch_conv_tiled(a, stream, shape);
     if (e != hipErrorNotSupported) return e;

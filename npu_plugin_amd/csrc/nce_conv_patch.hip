@@ -44,7 +44,7 @@ namespace {
 using namespace wres_detail;
 using namespace lds_detail;
 
-constexpr int kPatchWaves = 8;
+constexpr int kPatchWavesMax = 16;  // (probe builds size their trace by it)
 constexpr size_t kPatchLdsCap = 156 * 1024;  // dynamic LDS a workgroup may ask for (the per-channel tables are static)
 
 struct PatchArgs {
@@ -73,7 +73,7 @@ struct PatchArgs {
 static uint64_t* g_probe_trace = nullptr;  // set by the probe program before it launches
 #define PATCH_MARK(i)                                                                                                  \
     do {                                                                                                               \
-        if (lane == 0 && (i) < 32) w.trace[((size_t)blockIdx.x * kPatchWaves + wave) * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+        if (lane == 0 && (i) < 32) w.trace[((size_t)blockIdx.x * kPatchWavesMax + wave) * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
     } while (0)
 #define PATCH_MARK_DECL int patch_mark = 4
 #define PATCH_MARK_SEQ()  \
@@ -106,9 +106,11 @@ __device__ __forceinline__ int halo_piece(int key, int pos) {
     return (pos & ~15) | (2 * j + (pp >> (ULOG - 1)));
 }
 
-template <int NF, int NPX, int ULOG>
-__global__ __launch_bounds__(64 * kPatchWaves, 2) void conv_patch_kernel(PatchArgs w) {
-    constexpr int NW = kPatchWaves;
+// NW waves per workgroup: 8 with groups of NPX = 4 pixel fragments (two waves per SIMD, 256 registers each), or 16 with
+// groups of NPX = 2 (four waves per SIMD, 128 registers each: more waves to fill the matrix unit while others run their
+// epilogues or stand at a request, at 0.75 instead of 0.5 KiB of LDS reads per matrix instruction).
+template <int NF, int NPX, int ULOG, int NW>
+__global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w) {
     constexpr int BN = 16 * NF;
     const ConvArgs& a = w.a;
 
@@ -136,6 +138,12 @@ __global__ __launch_bounds__(64 * kPatchWaves, 2) void conv_patch_kernel(PatchAr
     if (p_begin >= p_end) return;  // uniform
 
     PATCH_MARK(0);
+#ifdef PATCH_PRIO
+    // The lower half of the waves (one or two per SIMD) outranks the upper half at instruction issue: where both are in
+    // their reductions the lower one gets the matrix unit and finishes at full speed, and the upper one runs its
+    // reduction while the lower one is in its epilogue - the two fall into opposite phases by themselves.
+    if (wave < NW / 2) __builtin_amdgcn_s_setprio(3);
+#endif
     const int wbytes = w.nsteps * NF * 1024;
     uint8_t* const sHalo = sL + wbytes;
     const int IC = a.IC;
@@ -372,7 +380,11 @@ __global__ __launch_bounds__(64 * kPatchWaves, 2) void conv_patch_kernel(PatchAr
 #pragma unroll
                 for (int x = 0; x < NPX; ++x) fb[x] = *reinterpret_cast<const v4i*>(hb + (abase[x] + tapoff + ((akq[x] + ts) & POSMASK)));
                 wp += NF * 1024;
+#ifdef PATCH_KO_WALK
+                if (false) {
+#else
                 if (++it_c == w.nc64) {
+#endif
                     it_c = 0;
                     if (++it_kx == a.KX) {
                         it_kx = 0;
@@ -386,41 +398,59 @@ __global__ __launch_bounds__(64 * kPatchWaves, 2) void conv_patch_kernel(PatchAr
 #pragma unroll
                     for (int x = 0; x < NPX; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[f], fb[x], acc[f][x], 0, 0, 0);
             };
-            v4i fa0[NF], fb0[NPX], fa1[NF], fb1[NPX];
             const int Sn = w.nsteps;
-            fetch(fa0, fb0);
-            if (Sn > 1) fetch(fa1, fb1);
-            {   // the first step starts the accumulators (no zeroing pass)
-                const v4i zero = {0, 0, 0, 0};
-#pragma unroll
-                for (int f = 0; f < NF; ++f)
-#pragma unroll
-                    for (int x = 0; x < NPX; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa0[f], fb0[x], zero, 0, 0, 0);
-            }
-            // (Both requests of the loop body are unconditional and the tail is written out, so that every block of matrix
-            // instructions follows the requests of the step after it on every path: the wait before it then names just
-            // the older set, and the younger one stays in flight.)
+            const v4i zero = {0, 0, 0, 0};
             auto request_one = [&]() {
+#ifdef PATCH_KO_NOREQ
+                if (false) {
+#else
                 if (kreq < w.nblk) {  // uniform
+#endif
                     request_block(nx, kreq);
                     kreq += NW;
                 }
             };
-            int s = 1;
-            for (; s + 2 < Sn; s += 2) {
+            if constexpr (NW == 8) {
+                // Two waves per SIMD: two register sets, so that the reads of step s + 1 are in flight while the matrix
+                // instructions of step s run. (Both requests of the loop body are unconditional and the tail is written out,
+                // so that every block of matrix instructions follows the requests of the step after it on every path: the
+                // wait before it then names just the older set, and the younger one stays in flight.)
+                v4i fa0[NF], fb0[NPX], fa1[NF], fb1[NPX];
                 fetch(fa0, fb0);
-                request_one();
-                mma(fa1, fb1);
-                fetch(fa1, fb1);
-                request_one();
-                mma(fa0, fb0);
-            }
-            if (s + 1 < Sn) {
+                if (Sn > 1) fetch(fa1, fb1);
+#pragma unroll
+                for (int f = 0; f < NF; ++f)  // the first step starts the accumulators (no zeroing pass)
+#pragma unroll
+                    for (int x = 0; x < NPX; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa0[f], fb0[x], zero, 0, 0, 0);
+                int s = 1;
+                for (; s + 2 < Sn; s += 2) {
+                    fetch(fa0, fb0);
+                    request_one();
+                    mma(fa1, fb1);
+                    fetch(fa1, fb1);
+                    request_one();
+                    mma(fa0, fb0);
+                }
+                if (s + 1 < Sn) {
+                    fetch(fa0, fb0);
+                    mma(fa1, fb1);
+                    mma(fa0, fb0);
+                } else if (s < Sn) {
+                    mma(fa1, fb1);
+                }
+            } else {
+                // Four waves per SIMD: one register set; the other waves cover this one's read latency.
+                v4i fa0[NF], fb0[NPX];
                 fetch(fa0, fb0);
-                mma(fa1, fb1);
-                mma(fa0, fb0);
-            } else if (s < Sn) {
-                mma(fa1, fb1);
+#pragma unroll
+                for (int f = 0; f < NF; ++f)
+#pragma unroll
+                    for (int x = 0; x < NPX; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa0[f], fb0[x], zero, 0, 0, 0);
+                for (int s = 1; s < Sn; ++s) {
+                    fetch(fa0, fb0);
+                    request_one();
+                    mma(fa0, fb0);
+                }
             }
             PATCH_MARK_SEQ();   // reduction done (issued)
             if (!next_done && g + NW >= ngr) finish_next();
@@ -466,29 +496,40 @@ __global__ __launch_bounds__(64 * kPatchWaves, 2) void conv_patch_kernel(PatchAr
     }
 }
 
-template <int NF, int NPX, int ULOG>
+template <int NF, int NPX, int ULOG, int NW>
 hipError_t launch_patch(const PatchArgs& w, size_t lds, hipStream_t stream) {
-    auto kernel = &conv_patch_kernel<NF, NPX, ULOG>;
+    auto kernel = &conv_patch_kernel<NF, NPX, ULOG, NW>;
     static LdsGrant grant;
     if (const hipError_t e = grant.ensure(reinterpret_cast<const void*>(kernel), lds, 48 * 1024); e != hipSuccess) return e;
     const uint32_t total = w.ngroups * w.nslices;
-    return emit(kernel, dim3(xcd_grid(total)), dim3(64 * kPatchWaves), lds, stream, w);
+    return emit(kernel, dim3(xcd_grid(total)), dim3(64 * NW), lds, stream, w);
 }
 
 template <int NF>
-hipError_t launch_patch_u(const PatchArgs& w, size_t lds, int ulog, hipStream_t stream) {
+hipError_t launch_patch_u(const PatchArgs& w, size_t lds, int ulog, int waves, hipStream_t stream) {
+    if (waves == 16) {
+        switch (ulog) {
+        case 2: return launch_patch<NF, 2, 2, 16>(w, lds, stream);
+        case 3: return launch_patch<NF, 2, 3, 16>(w, lds, stream);
+        case 4: return launch_patch<NF, 2, 4, 16>(w, lds, stream);
+        default: return hipErrorNotSupported;
+        }
+    }
     switch (ulog) {
-    case 2: return launch_patch<NF, 4, 2>(w, lds, stream);
-    case 3: return launch_patch<NF, 4, 3>(w, lds, stream);
-    case 4: return launch_patch<NF, 4, 4>(w, lds, stream);
+    case 2: return launch_patch<NF, 4, 2, 8>(w, lds, stream);
+    case 3: return launch_patch<NF, 4, 3, 8>(w, lds, stream);
+    case 4: return launch_patch<NF, 4, 4, 8>(w, lds, stream);
     default: return hipErrorNotSupported;
     }
 }
 
 }  // namespace
 
-// nf_forced: 0 = automatic, 2 or 4 = channel fragments per slice; pr_forced: 0 = automatic, else output rows per patch.
-hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_forced, int pr_forced) {
+// nf_forced: 0 = automatic, 2 or 4 = channel fragments per slice; pr_forced: 0 = automatic, else output rows per patch;
+// waves_forced: 0 = automatic, 8 or 16 = waves per workgroup (groups of four or two pixel fragments).
+hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_forced, int pr_forced, int waves_forced) {
+    const int waves = waves_forced == 16 ? 16 : 8;
+    const int npxf = waves == 16 ? 2 : 4;  // pixel fragments per group
     if (a.SY != 1 || a.SX != 1 || a.dw != 0) return hipErrorNotSupported;
     if (a.IC != 64 && a.IC != 128 && a.IC != 256 && a.IC != 512 && a.IC != 1024) return hipErrorNotSupported;
     if (a.KY > 16 || a.KX > 16 || a.bw > 4096 || a.bh > 32768) return hipErrorNotSupported;
@@ -539,8 +580,8 @@ hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_force
             const int64_t np = nimg * ((a.bh + cand - 1) / cand);
             const int64_t groups = std::min<int64_t>(np, std::max<int64_t>(1, cus / (int64_t)w.nslices));
             const int64_t tpg = (np + groups - 1) / groups;
-            const int64_t ngr = (((int64_t)cand * a.bw + 15) / 16 + 3) / 4;
-            double cost = (double)tpg * ((double)((ngr + 3) / 4) + 0.5);
+            const int64_t ngr = (((int64_t)cand * a.bw + 15) / 16 + npxf - 1) / npxf;
+            double cost = (double)tpg * ((double)((ngr + 3) / 4) * (npxf / 4.0) + 0.5);
             if (tpg > 1 && wbytes(nf) + 2 * halo_bytes(cand) > kPatchLdsCap) cost *= 1.15;
             if (pr == 0 || cost <= best) {
                 best = cost;
@@ -571,10 +612,10 @@ hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_force
     w.trace = g_probe_trace;
 #endif
     if (tls_launch.log != nullptr)
-        tls_launch.log->add(3, "conv: patch kernel, %d channels per slice, %d rows per patch, %d patch buffer(s), %u workgroups x %u patches",
-                            16 * nf, w.PR, w.nbuf, w.ngroups * w.nslices, w.tpg);
-    if (nf == 4) return launch_patch_u<4>(w, lds, ulog, stream);
-    return launch_patch_u<2>(w, lds, ulog, stream);
+        tls_launch.log->add(3, "conv: patch kernel, %d channels per slice, %d rows per patch, %d patch buffer(s), %u workgroups of %d waves x %u patches",
+                            16 * nf, w.PR, w.nbuf, w.ngroups * w.nslices, waves, w.tpg);
+    if (nf == 4) return launch_patch_u<4>(w, lds, ulog, waves, stream);
+    return launch_patch_u<2>(w, lds, ulog, waves, stream);
 }
 
 }  // namespace nce

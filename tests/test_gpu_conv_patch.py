@@ -36,7 +36,7 @@ def _id(s):
     return f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}"
 
 
-@pytest.mark.parametrize("knob", ["1", "4,1", "4,3", "2,5", "2,64"])
+@pytest.mark.parametrize("knob", ["1", "4,1", "4,3", "2,5", "2,64", "4,3,16", "2,6,16"])
 @pytest.mark.parametrize("shape", PATCH_SHAPES, ids=_id)
 def test_conv_patch_shapes(tuned, shape, knob):
     n, h, w, ic, oc, k, pads, in_zp = shape
@@ -45,7 +45,7 @@ def test_conv_patch_shapes(tuned, shape, knob):
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
 
 
-@pytest.mark.parametrize("knob", ["1", "4,2", "2,3"])
+@pytest.mark.parametrize("knob", ["1", "4,2", "2,3", "4,2,16"])
 def test_conv_patch_types_and_modes(tuned, knob):
     executor = tuned(NCE_HIP_CONV_PATCH=knob)
     wide = dict(k=(3, 3), pads=(1, 1, 1, 1))
