@@ -94,6 +94,46 @@ nce_result_t nceHwtestBuildTask(nce_hwtest_case_handle_t hw_case, nce_cluster_ta
                                 nce_ppe_task_t* ppe, int32_t* table, int32_t table_capacity_rows, int32_t* table_rows,
                                 nce_log_handle_t log);
 
+/* Case types that the reference builds as several NCE tasks (one program per case):
+ *   DoubleZMajorConvolution  two chained convolutions through a tensor of the output's type (buildDoubleConvTest.cpp:55-492)
+ *   RaceConditionDPU         the same convolution on num_clusters clusters, iteration_count times each; every cluster's
+ *                            output must hold the same bytes (buildRaceConditionDPUTest.cpp:41-243)
+ *   DifferentClustersDPU     one convolution whose output goes to every cluster of DPUTaskParams.output_cluster
+ *                            (buildDIfferentClustersDPUTest.cpp:25-260)
+ *   MultiClustersDPU         one convolution split over DPUTaskParams.task_clusters along the rows (SOH) or the output
+ *                            channels (SOK), each cluster one workload (buildMultiClustersDPUTest.cpp:289-626)
+ * None of them adds a PPE task. A GPU has no clusters: a "cluster" is one output tensor and, for MultiClustersDPU, one
+ * workload (variant) whose cluster_id names it. */
+#define NCE_HWTEST_MAX_OUTPUTS 8
+
+typedef struct nce_hwtest_program_t {
+    int32_t num_tasks;          /* tasks to run, in order, on one stream (what the program's barriers encode) */
+    int32_t num_outputs;        /* tensors the program returns: one per cluster where the case names clusters */
+    int32_t num_intermediates;  /* 1 for DoubleZMajorConvolution (the first convolution's output), else 0 */
+    int32_t outputs_identical;  /* 1: every output must hold the same bytes */
+    int64_t output_shape[NCE_HWTEST_MAX_OUTPUTS][4]; /* logical N, C, H, W of each output (type: the case's output) */
+    int64_t intermediate_shape[4];                   /* dense NHWC, the output's type and zero point */
+} nce_hwtest_program_t;
+
+/* Which tensors task `index` reads and writes. The descriptor's data pointers are NULL; the caller sets
+ * input.data = base of the input tensor + input_offset_bytes, output.data = base of the output tensor +
+ * output_offset_bytes, weights.data = the weights of entry weight_layer of "weight" + weights_offset_bytes. The offsets
+ * are non-zero where a cluster computes a slice into a tensor of its own (MultiClustersDPU without broadcast): the task
+ * is then the convolution over the input rows / the weights rows that slice needs. */
+typedef struct nce_hwtest_binding_t {
+    int32_t input_tensor;   /* -1: the case's input; 0: the intermediate tensor */
+    int32_t output_tensor;  /* >= 0: output of that index; -1: the intermediate tensor */
+    int32_t weight_layer;   /* entry of "weight" */
+    int32_t reserved;
+    int64_t input_offset_bytes, output_offset_bytes, weights_offset_bytes;
+} nce_hwtest_binding_t;
+
+nce_result_t nceHwtestGetProgram(nce_hwtest_case_handle_t hw_case, nce_hwtest_program_t* out, nce_log_handle_t log);
+/* nceHwtestBuildTask for task `index` of the case's program (index 0 of a single-task case is that task). */
+nce_result_t nceHwtestBuildTaskAt(nce_hwtest_case_handle_t hw_case, int32_t index, nce_cluster_task_desc_t* desc,
+                                  nce_dpu_task_t* variant, nce_ppe_task_t* ppe, int32_t* table, int32_t table_capacity_rows,
+                                  int32_t* table_rows, nce_hwtest_binding_t* binding, nce_log_handle_t log);
+
 #ifdef __cplusplus
 }
 #endif

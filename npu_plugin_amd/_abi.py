@@ -135,6 +135,32 @@ class HwtestLayer(C.Structure):
     ]
 
 
+HWTEST_MAX_OUTPUTS = 8
+
+
+class HwtestProgram(C.Structure):
+    _fields_ = [
+        ("num_tasks", C.c_int32),
+        ("num_outputs", C.c_int32),
+        ("num_intermediates", C.c_int32),
+        ("outputs_identical", C.c_int32),
+        ("output_shape", (C.c_int64 * 4) * HWTEST_MAX_OUTPUTS),
+        ("intermediate_shape", C.c_int64 * 4),
+    ]
+
+
+class HwtestBinding(C.Structure):
+    _fields_ = [
+        ("input_tensor", C.c_int32),
+        ("output_tensor", C.c_int32),
+        ("weight_layer", C.c_int32),
+        ("reserved", C.c_int32),
+        ("input_offset_bytes", C.c_int64),
+        ("output_offset_bytes", C.c_int64),
+        ("weights_offset_bytes", C.c_int64),
+    ]
+
+
 class HwtestCase(C.Structure):
     _fields_ = [
         ("arch", C.c_int32),
@@ -225,6 +251,9 @@ SYMBOLS = {
     "nceVpuipEnqueue": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "nceHwtestBuildTask": (C.c_int, [C.c_void_p, _P(ClusterTaskDesc), _P(DpuTask), _P(PpeTask), _P(C.c_int32), C.c_int32,
                                      _P(C.c_int32), C.c_void_p]),
+    "nceHwtestGetProgram": (C.c_int, [C.c_void_p, _P(HwtestProgram), C.c_void_p]),
+    "nceHwtestBuildTaskAt": (C.c_int, [C.c_void_p, C.c_int32, _P(ClusterTaskDesc), _P(DpuTask), _P(PpeTask), _P(C.c_int32),
+                                       C.c_int32, _P(C.c_int32), _P(HwtestBinding), C.c_void_p]),
 }
 
 _lib = None

@@ -44,7 +44,6 @@ namespace {
 using namespace wres_detail;
 using namespace lds_detail;
 
-constexpr int kPatchWavesMax = 16;  // (probe builds size their trace by it)
 constexpr size_t kPatchLdsCap = 156 * 1024;  // dynamic LDS a workgroup may ask for (the per-channel tables are static)
 
 struct PatchArgs {
@@ -73,7 +72,7 @@ struct PatchArgs {
 static uint64_t* g_probe_trace = nullptr;  // set by the probe program before it launches
 #define PATCH_MARK(i)                                                                                                  \
     do {                                                                                                               \
-        if (lane == 0 && (i) < 32) w.trace[((size_t)blockIdx.x * kPatchWavesMax + wave) * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+        if (lane == 0 && (i) < 32) w.trace[((size_t)blockIdx.x * 16 + wave) * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
     } while (0)
 #define PATCH_MARK_DECL int patch_mark = 4
 #define PATCH_MARK_SEQ()  \

@@ -298,10 +298,21 @@ struct Layer {
 
 }  // namespace
 
+// Case types that expand to several NCE tasks (include/nce_hwtest.h, nce_hwtest_program_t).
+enum ProgramKind { PROGRAM_SINGLE = 0, PROGRAM_DOUBLE_CONV, PROGRAM_RACE_DPU, PROGRAM_DIFFERENT_CLUSTERS, PROGRAM_MULTI_CLUSTERS };
+
 struct nce_hwtest_case_s {
     nce_hwtest_case_t pub{};
     Layer in, wt, out;
     bool has_conv = false, has_pool = false, has_ew = false;
+    int program = PROGRAM_SINGLE;
+    Layer wt2;                          // DoubleZMajorConvolution: second entry of "weight"
+    std::vector<Layer> outs;            // every entry of "output" (MultiClustersDPU: one per cluster)
+    int64_t iteration_count = 1;        // RaceConditionDPU
+    int64_t num_clusters = 1;           // RaceConditionDPU
+    std::vector<int64_t> clusters;      // DifferentClustersDPU: output_cluster; MultiClustersDPU: task_clusters
+    int split_dim = 0;                  // MultiClustersDPU: 1 = SOK (channels), 2 = SOH (rows)
+    bool broadcast = false;             // MultiClustersDPU
 };
 
 namespace {
@@ -338,10 +349,15 @@ void load_quant(const JValue& obj, const char* who, Layer* l) {
 }
 
 // loadInputLayer / loadWeightLayer / loadOutputLayer, :464-585: arrays of objects; the first entry is the operand.
-void load_layer(const JValue& root, const char* key, const char* missing_shape, Layer* l) {
+size_t layer_count(const JValue& root, const char* key) {
     const JArray* arr = root.getArray(key);
-    if (!arr || arr->empty()) return;
-    const JValue& obj = (*arr)[0];
+    return arr ? arr->size() : 0;
+}
+
+void load_layer(const JValue& root, const char* key, const char* missing_shape, Layer* l, size_t index = 0) {
+    const JArray* arr = root.getArray(key);
+    if (!arr || arr->size() <= index) return;
+    const JValue& obj = (*arr)[index];
     if (obj.kind != JValue::Object) throw std::runtime_error(std::string(key) + ": entries must be objects");
     const JArray* shape = obj.getArray("shape");
     if (!shape) bad(missing_shape);
@@ -491,6 +507,70 @@ void parse_case(const std::string& text, nce_hwtest_case_s* c) {
         c->pub.task_type = NCE_TASK_ELTWISE;
         load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt);
         load_eltwise(root, c);
+    } else if (iequal(case_type, "DoubleZMajorConvolution")) {
+        // two chained convolutions (buildDoubleConvTest.cpp:55-492); parse: test_case_json_parser.cpp:887-908
+        c->pub.task_type = NCE_TASK_CONV;
+        c->program = PROGRAM_DOUBLE_CONV;
+        load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt);
+        load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt2, 1);
+        if (!c->wt2.pub.present) bad("DoubleZMajorConvolution: the weight list needs two entries");
+        load_conv(root, c);
+        load_output_order(root, c);
+    } else if (iequal(case_type, "RaceConditionDPU")) {
+        // the same convolution on num_clusters clusters, iteration_count times each; every cluster's output must hold the
+        // same bytes (buildRaceConditionDPUTest.cpp:41-243); parse: :909-915, loadIterationCount / loadNumClusters :783-794
+        c->pub.task_type = NCE_TASK_CONV;
+        c->program = PROGRAM_RACE_DPU;
+        load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt);
+        load_conv(root, c);
+        if (!root.getInteger("iteration_count", &c->iteration_count) || c->iteration_count < 1) bad("RaceConditionDPU: iteration_count must be a positive integer");
+        if (!root.getInteger("num_clusters", &c->num_clusters) || c->num_clusters < 1) bad("RaceConditionDPU: num_clusters must be a positive integer");
+    } else if (iequal(case_type, "DifferentClustersDPU")) {
+        // one convolution whose operands sit in the CMX of different clusters and whose output goes to every cluster of
+        // output_cluster (buildDIfferentClustersDPUTest.cpp:25-260); parse: loadDPUTaskParams, :417-434
+        c->pub.task_type = NCE_TASK_CONV;
+        c->program = PROGRAM_DIFFERENT_CLUSTERS;
+        load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt);
+        load_conv(root, c);
+        const JValue* tp = root.getObjectValue("DPUTaskParams");
+        const JArray* oc = tp ? tp->getArray("output_cluster") : nullptr;
+        if (!oc) bad("loadDPUTaskParams: cannot find output_cluster config param");
+        for (const JValue& e : *oc) {
+            int64_t v;
+            if (e.asInteger(&v)) c->clusters.push_back(v);
+        }
+        int64_t v;
+        if (!tp->getInteger("input_cluster", &v) || !tp->getInteger("weights_cluster", &v) || !tp->getInteger("weights_table_cluster", &v))
+            bad("loadDPUTaskParams: input_cluster, weights_cluster and weights_table_cluster are required");
+        if (c->clusters.empty()) bad("loadDPUTaskParams: output_cluster is empty");
+    } else if (iequal(case_type, "MultiClustersDPU")) {
+        // one convolution split over clusters along the rows (SOH) or the output channels (SOK)
+        // (buildMultiClustersDPUTest.cpp:289-626); parse: loadMultiClusterDPUParams, :436-459
+        c->pub.task_type = NCE_TASK_CONV;
+        c->program = PROGRAM_MULTI_CLUSTERS;
+        load_layer(root, "weight", "loadWeightLayer: missing shape", &c->wt);
+        load_conv(root, c);
+        load_output_order(root, c);
+        const JValue* tp = root.getObjectValue("DPUTaskParams");
+        const JArray* tc = tp ? tp->getArray("task_clusters") : nullptr;
+        if (!tc) bad("loadMultiClusterDPUParams: cannot find task_clusters config param");
+        for (const JValue& e : *tc) {
+            int64_t v;
+            if (e.asInteger(&v)) c->clusters.push_back(v);
+        }
+        std::string seg;
+        if (!tp->getString("segmentation", &seg) || (seg != "SOK" && seg != "SOH")) bad("loadMultiClusterDPUParams: failed to get valid segmentation type");
+        c->split_dim = seg == "SOK" ? 1 : 2;  // (SegmentationType's value is the dimension split: C = 1, H = 2)
+        bool b = false;
+        if (!tp->getBoolean("broadcast", &b)) bad("loadMultiClusterDPUParams: broadcast is required");
+        c->broadcast = b;
+        if (c->clusters.empty()) bad("loadMultiClusterDPUParams: task_clusters is empty");
+        for (size_t i = 0; i < layer_count(root, "output"); ++i) {
+            Layer l;
+            load_layer(root, "output", "loadOutputLayer: missing shape", &l, i);
+            c->outs.push_back(l);
+        }
+        if (c->outs.size() != c->clusters.size()) bad("MultiClustersDPU: one output entry per task cluster is required");
     } else if (iequal(case_type, "MaxPool")) {
         c->pub.task_type = NCE_TASK_MAXPOOL;
         load_pool(root, c);
@@ -498,11 +578,11 @@ void parse_case(const std::string& text, nce_hwtest_case_s* c) {
         c->pub.task_type = NCE_TASK_AVEPOOL;
         load_pool(root, c);
     } else {
-        static const char* other[] = {"DMA", "DMAcompressAct", "SparseZMajorConvolution", "DoubleZMajorConvolution",
-                                      "EltwiseMultDW", "EltwiseSparse", "DifferentClustersDPU", "MultiClustersDPU",
+        static const char* other[] = {"DMA", "DMAcompressAct", "SparseZMajorConvolution",
+                                      "EltwiseMultDW", "EltwiseSparse",
                                       "ActShave", "ReadAfterWriteDPUDMA", "ReadAfterWriteDMADPU", "ReadAfterWriteACTDMA",
                                       "ReadAfterWriteDMAACT", "ReadAfterWriteDPUACT", "ReadAfterWriteACTDPU",
-                                      "RaceConditionDMA", "RaceConditionDPU", "RaceConditionDPUDMA",
+                                      "RaceConditionDMA", "RaceConditionDPUDMA",
                                       "RaceConditionDPUDMAACT", "RaceConditionDPUACT", "RaceCondition",
                                       "StorageElementTableDPU", "DualChannelDMA", "GenerateScaleTable"};
         bool known = false;
@@ -787,6 +867,207 @@ void build(const nce_hwtest_case_s& c, nce_cluster_task_desc_t* d, nce_dpu_task_
     }
 }
 
+
+// ---- case types that expand to several tasks ---------------------------------------------------------
+
+int64_t conv_out(int64_t in, int64_t k, int64_t pad_a, int64_t pad_b, int64_t stride) {
+    return (in - k + pad_a + pad_b) / stride + 1;
+}
+
+// Rows (SOH) or channels (SOK) each cluster computes. Without broadcast the case lists one output per cluster and the
+// sizes are theirs (buildMultiClustersDPUTest.cpp:306-321); with broadcast every entry has the whole shape and the split
+// is the even one of the distributed output type: ceil(size / clusters) per cluster, channels in multiples of 16
+// (DistributedAttrs, :36-93) - the last cluster takes what is left.
+std::vector<int64_t> cluster_sizes(const nce_hwtest_case_s& c, int64_t parent) {
+    const size_t n = c.clusters.size();
+    std::vector<int64_t> sizes(n, 0);
+    if (!c.broadcast) {
+        for (size_t i = 0; i < n; ++i) sizes[i] = c.outs[i].pub.shape[c.split_dim];
+        return sizes;
+    }
+    int64_t per = (parent + (int64_t)n - 1) / (int64_t)n;
+    if (c.split_dim == 1) per = (per + 15) / 16 * 16;
+    int64_t left = parent;
+    for (size_t i = 0; i < n; ++i) {
+        sizes[i] = std::max<int64_t>(0, std::min(per, left));
+        left -= sizes[i];
+    }
+    return sizes;
+}
+
+void parent_output_shape(const nce_hwtest_case_s& c, int64_t (&shape)[4]) {
+    for (int i = 0; i < 4; ++i) shape[i] = c.pub.output.shape[i];
+    if (c.program == PROGRAM_MULTI_CLUSTERS && !c.broadcast)
+        for (size_t k = 1; k < c.outs.size(); ++k) shape[c.split_dim] += c.outs[k].pub.shape[c.split_dim];
+}
+
+void program_of(const nce_hwtest_case_s& c, nce_hwtest_program_t* g) {
+    memset(g, 0, sizeof(*g));
+    const nce_hwtest_case_t& p = c.pub;
+    g->num_tasks = 1;
+    g->num_outputs = 1;
+    for (int i = 0; i < 4; ++i) g->output_shape[0][i] = p.output.shape[i];
+    auto outputs = [&](size_t n) {
+        if (n > NCE_HWTEST_MAX_OUTPUTS) throw Unsupported("more clusters than this front end describes (" + std::to_string(NCE_HWTEST_MAX_OUTPUTS) + ")");
+        g->num_outputs = (int32_t)n;
+        for (size_t k = 0; k < n; ++k)
+            for (int i = 0; i < 4; ++i) g->output_shape[k][i] = p.output.shape[i];
+    };
+    switch (c.program) {
+    case PROGRAM_DOUBLE_CONV:
+        g->num_tasks = 2;
+        g->num_intermediates = 1;
+        g->intermediate_shape[0] = p.input.shape[0];
+        g->intermediate_shape[1] = p.weight.shape[0];
+        g->intermediate_shape[2] = conv_out(p.input.shape[2], p.weight.shape[2], p.pad[0], p.pad[2], std::max(1, p.stride[0]));
+        g->intermediate_shape[3] = conv_out(p.input.shape[3], p.weight.shape[3], p.pad[1], p.pad[3], std::max(1, p.stride[1]));
+        break;
+    case PROGRAM_RACE_DPU:
+        outputs((size_t)c.num_clusters);
+        if (c.iteration_count * c.num_clusters > 1 << 20) throw Unsupported("iteration_count x num_clusters is too large");
+        g->num_tasks = (int32_t)(c.iteration_count * c.num_clusters);
+        g->outputs_identical = 1;
+        break;
+    case PROGRAM_DIFFERENT_CLUSTERS:
+        outputs(c.clusters.size());
+        g->num_tasks = g->num_outputs;
+        g->outputs_identical = 1;
+        break;
+    case PROGRAM_MULTI_CLUSTERS: {
+        const size_t n = c.clusters.size();
+        outputs(n);
+        if (c.broadcast) {  // every cluster's buffer receives every slice
+            g->num_tasks = (int32_t)(n * n);
+            g->outputs_identical = 1;
+        } else {
+            g->num_tasks = (int32_t)n;
+            for (size_t k = 0; k < n; ++k)
+                for (int i = 0; i < 4; ++i) g->output_shape[k][i] = c.outs[k].pub.shape[i];
+        }
+        break;
+    }
+    default: break;
+    }
+}
+
+// Task `index` of a case. Single-task cases: index 0 is nceHwtestBuildTask's task.
+void build_at(const nce_hwtest_case_s& c, int32_t index, nce_cluster_task_desc_t* d, nce_dpu_task_t* var, nce_ppe_task_t* ppe,
+              int32_t* table, int32_t cap_rows, int32_t* rows, nce_hwtest_binding_t* bind) {
+    nce_hwtest_program_t g;
+    program_of(c, &g);
+    if (index < 0 || index >= g.num_tasks) throw std::runtime_error("task index out of range");
+    memset(bind, 0, sizeof(*bind));
+    bind->input_tensor = -1;
+    if (c.program == PROGRAM_SINGLE) {
+        build(c, d, var, ppe, table, cap_rows, rows);
+        return;
+    }
+    // These builders add no PPE task and take no activation (only buildZMConvTest.cpp does): NOOP, storage-range clamp.
+    if (c.pub.activation != NCE_HWTEST_ACT_NONE) throw Unsupported(std::string("case type '") + c.pub.case_type + "' takes no activation");
+    nce_hwtest_case_s one = c;  // the convolution this task is, as a single-task case
+    one.program = PROGRAM_SINGLE;
+    switch (c.program) {
+    case PROGRAM_DOUBLE_CONV: {
+        // Both convolutions share kernel size (taken from the first weights), strides and paddings, and both weights tables
+        // are computed from the case's input, first-weights and output types (buildDoubleConvTest.cpp:329-360,
+        // hwtest.cpp:114: weightTypes.front()); the tensor between them has the output's type and is dense NHWC.
+        if (c.wt2.pub.shape[2] != c.wt.pub.shape[2] || c.wt2.pub.shape[3] != c.wt.pub.shape[3])
+            throw Unsupported("DoubleZMajorConvolution: both weights must have the kernel size of the first");
+        if (index == 0) {
+            for (int i = 0; i < 4; ++i) one.pub.output.shape[i] = one.out.pub.shape[i] = g.intermediate_shape[i];
+            copy_str(one.pub.output_order, sizeof(one.pub.output_order), "nhwc");
+            bind->output_tensor = -1;
+        } else {
+            if (c.wt2.pub.shape[1] != g.intermediate_shape[1]) throw std::runtime_error("second weights' input channels differ from the first weights' output channels");
+            one.in.pub.dtype = c.out.pub.dtype;
+            one.in.pub.zero_point = c.out.pub.zero_point;
+            copy_str(one.in.pub.dtype_name, sizeof(one.in.pub.dtype_name), c.out.pub.dtype_name);
+            for (int i = 0; i < 4; ++i) one.in.pub.shape[i] = g.intermediate_shape[i];
+            one.pub.input = one.in.pub;
+            for (int i = 0; i < 4; ++i) one.wt.pub.shape[i] = c.wt2.pub.shape[i];  // (type and scales stay the first weights')
+            one.pub.weight = one.wt.pub;
+            bind->input_tensor = 0;
+            bind->weight_layer = 1;
+        }
+        build(one, d, var, ppe, table, cap_rows, rows);
+        break;
+    }
+    case PROGRAM_RACE_DPU:
+        // iteration i runs the task once per cluster (buildRaceConditionDPUTest.cpp:135-215)
+        build(one, d, var, ppe, table, cap_rows, rows);
+        bind->output_tensor = index % (int32_t)c.num_clusters;
+        var->cluster_id = bind->output_tensor;
+        break;
+    case PROGRAM_DIFFERENT_CLUSTERS:
+        build(one, d, var, ppe, table, cap_rows, rows);
+        bind->output_tensor = index;
+        var->cluster_id = (int32_t)c.clusters[(size_t)index];
+        break;
+    case PROGRAM_MULTI_CLUSTERS: {
+        // Cluster `slice` computes its rows or channels of the parent output (:543-581; paddings per cluster as
+        // getMulticlusteringPaddings, hwtest_utils.cpp:527-597). With broadcast every cluster's output tensor is the whole
+        // parent: the task is the whole convolution with ONE workload, the slice's box. Without broadcast the cluster's own
+        // tensor holds just the slice, and the task is the convolution that produces it on its own: the slice's weights
+        // and table rows (channels), or the input rows the slice reads with the paddings that remain (rows); the binding
+        // says where in the case's weights / input that view starts.
+        const int32_t n = (int32_t)c.clusters.size();
+        const int32_t slice = c.broadcast ? index % n : index;
+        int64_t parent[4];
+        parent_output_shape(c, parent);
+        const std::vector<int64_t> sizes = cluster_sizes(c, parent[c.split_dim]);
+        int64_t start = 0;
+        for (int32_t k = 0; k < slice; ++k) start += sizes[(size_t)k];
+        const int64_t size = sizes[(size_t)slice];
+        if (size <= 0 || start + size > parent[c.split_dim]) throw std::runtime_error("MultiClustersDPU: cluster slices do not fit the output");
+        // effective paddings and input rows of output rows [start, start + size)
+        const int64_t sy = std::max(1, c.pub.stride[0]), IH = c.pub.input.shape[2], KY = c.pub.weight.shape[2];
+        const int64_t first = start * sy - c.pub.pad[0], last = (start + size - 1) * sy - c.pub.pad[0] + KY - 1;
+        const int64_t pad_top = std::max<int64_t>(0, -first), pad_bottom = std::max<int64_t>(0, last - (IH - 1));
+        for (int i = 0; i < 4; ++i) one.pub.output.shape[i] = one.out.pub.shape[i] = parent[i];
+        if (c.broadcast) {
+            build(one, d, var, ppe, table, cap_rows, rows);
+            const int box = c.split_dim == 1 ? 2 : 1;  // out_start / out_end are (x, y, z)
+            var->out_start[box] = (int32_t)start;
+            var->out_end[box] = (int32_t)(start + size - 1);
+            if (c.split_dim == 2) {
+                var->pad_top = (int32_t)pad_top;
+                var->pad_bottom = (int32_t)pad_bottom;
+            }
+            bind->output_tensor = index / n;
+        } else {
+            one.pub.output.shape[c.split_dim] = one.out.pub.shape[c.split_dim] = size;
+            if (c.split_dim == 1) {
+                one.pub.weight.shape[0] = one.wt.pub.shape[0] = size;
+                auto cut = [&](std::vector<double>* v) {
+                    if (v->size() > 1) {
+                        if ((int64_t)v->size() != parent[1]) throw std::runtime_error("per-channel scale count does not match the output channels");
+                        *v = std::vector<double>(v->begin() + start, v->begin() + start + size);
+                    }
+                };
+                cut(&one.wt.scales);
+                cut(&one.out.scales);
+                build(one, d, var, ppe, table, cap_rows, rows);
+                bind->weights_offset_bytes = start * d->weights.strides_bytes[0];
+            } else {
+                const int64_t r0 = std::max<int64_t>(0, first), r1 = std::min(IH - 1, last);
+                if (r1 < r0) throw std::runtime_error("MultiClustersDPU: a cluster's rows read no input row");
+                one.pub.input.shape[2] = one.in.pub.shape[2] = r1 - r0 + 1;
+                one.pub.pad[0] = (int32_t)pad_top;
+                one.pub.pad[2] = (int32_t)pad_bottom;
+                build(one, d, var, ppe, table, cap_rows, rows);
+                const int64_t row_bytes = d->input.strides_bytes[2];
+                d->input.strides_bytes[0] = IH * row_bytes;  // a view of the case's input
+                bind->input_offset_bytes = r0 * row_bytes;
+            }
+            bind->output_tensor = slice;
+        }
+        var->cluster_id = (int32_t)c.clusters[(size_t)slice];
+        break;
+    }
+    default: throw Unsupported("unknown program kind");
+    }
+}
+
 void log_error(nce_log_handle_t log, const char* what) {
     if (log != nullptr) log->add(1, "hwtest: %s", what);
 }
@@ -840,7 +1121,42 @@ nce_result_t nceHwtestBuildTask(nce_hwtest_case_handle_t hw_case, nce_cluster_ta
     if (hw_case == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
     if (desc == nullptr || variant == nullptr || ppe == nullptr || table_rows == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
     try {
-        build(*hw_case, desc, variant, ppe, table, table_capacity_rows, table_rows);
+        nce_hwtest_binding_t binding;
+        build_at(*hw_case, 0, desc, variant, ppe, table, table_capacity_rows, table_rows, &binding);
+        return NCE_RESULT_SUCCESS;
+    } catch (const Unsupported& e) {
+        log_error(log, e.what());
+        return NCE_RESULT_ERROR_UNSUPPORTED;
+    } catch (const std::bad_alloc&) {
+        return NCE_RESULT_ERROR_OUT_OF_MEMORY;
+    } catch (const std::exception& e) {
+        log_error(log, e.what());
+        return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    }
+}
+
+nce_result_t nceHwtestGetProgram(nce_hwtest_case_handle_t hw_case, nce_hwtest_program_t* out, nce_log_handle_t log) {
+    if (hw_case == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (out == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    try {
+        program_of(*hw_case, out);
+        return NCE_RESULT_SUCCESS;
+    } catch (const Unsupported& e) {
+        log_error(log, e.what());
+        return NCE_RESULT_ERROR_UNSUPPORTED;
+    } catch (const std::exception& e) {
+        log_error(log, e.what());
+        return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    }
+}
+
+nce_result_t nceHwtestBuildTaskAt(nce_hwtest_case_handle_t hw_case, int32_t index, nce_cluster_task_desc_t* desc, nce_dpu_task_t* variant,
+                                  nce_ppe_task_t* ppe, int32_t* table, int32_t table_capacity_rows, int32_t* table_rows,
+                                  nce_hwtest_binding_t* binding, nce_log_handle_t log) {
+    if (hw_case == nullptr) return NCE_RESULT_ERROR_INVALID_NULL_HANDLE;
+    if (desc == nullptr || variant == nullptr || ppe == nullptr || table_rows == nullptr || binding == nullptr) return NCE_RESULT_ERROR_INVALID_ARGUMENT;
+    try {
+        build_at(*hw_case, index, desc, variant, ppe, table, table_capacity_rows, table_rows, binding);
         return NCE_RESULT_SUCCESS;
     } catch (const Unsupported& e) {
         log_error(log, e.what());

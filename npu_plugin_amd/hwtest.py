@@ -82,6 +82,66 @@ class HwtestCase:
         task.finalize()
         return task
 
+    def program(self, executor=None):
+        """(num_tasks, output shapes, intermediate shape or None, outputs_identical) of the case's program: the case types
+        the reference builds as several NCE tasks (DoubleZMajorConvolution, RaceConditionDPU, DifferentClustersDPU,
+        MultiClustersDPU); a single-task case is a program of one task and one output."""
+        g = abi.HwtestProgram()
+        log = executor._log if executor is not None else None
+        rc = self._lib.nceHwtestGetProgram(self._handle, C.byref(g), log)
+        if rc != abi.SUCCESS:
+            raise NCEError(rc, executor.log() if executor is not None else "")
+        outs = [tuple(int(v) for v in g.output_shape[k]) for k in range(g.num_outputs)]
+        mid = tuple(int(v) for v in g.intermediate_shape) if g.num_intermediates else None
+        return g.num_tasks, outs, mid, bool(g.outputs_identical)
+
+    def build_program(self, input, weights, outputs, intermediate=None, executor=None):
+        """The case's tasks in program order. `weights`: one buffer per entry of the case's "weight" list; `outputs`: one
+        buffer per output of program() (memory order: the case's output_order); `intermediate`: the tensor between the two
+        convolutions of a DoubleZMajorConvolution (NHWC). Buffers are torch tensors or numpy arrays."""
+        num_tasks, _, _, _ = self.program(executor)
+        if not isinstance(weights, (list, tuple)):
+            weights = [weights]
+        tasks = []
+        log = executor._log if executor is not None else None
+        oc_max = max([int(self.info.output.shape[1]), int(self.info.weight.shape[0])] + [int(w.shape[0]) for w in weights if w is not None])
+        for index in range(num_tasks):
+            desc = abi.ClusterTaskDesc()
+            variant = abi.DpuTask()
+            ppe = abi.PpeTask()
+            bind = abi.HwtestBinding()
+            table = np.zeros((max(oc_max, 1), 4), dtype=np.int32)
+            rows = C.c_int32(0)
+            rc = self._lib.nceHwtestBuildTaskAt(self._handle, index, C.byref(desc), C.byref(variant), C.byref(ppe),
+                                                table.ctypes.data_as(C.POINTER(C.c_int32)), oc_max, C.byref(rows), C.byref(bind), log)
+            if rc != abi.SUCCESS:
+                raise NCEError(rc, executor.log() if executor is not None else "")
+            src = input if bind.input_tensor < 0 else intermediate
+            dst = outputs[bind.output_tensor] if bind.output_tensor >= 0 else intermediate
+            wts = weights[bind.weight_layer]
+            if src is None or dst is None:
+                raise ValueError("this case needs an intermediate tensor (see program())")
+            task = NCEClusterTask(desc.task_type, None)
+            task.desc = desc
+            task._variants = [variant]
+            task._ppe = ppe
+            task.table = table[:rows.value] if rows.value else None
+            task.binding = bind
+            task._keep = [src, wts, dst]
+            desc.input.data = _address(src) + bind.input_offset_bytes
+            desc.output.data = _address(dst) + bind.output_offset_bytes
+            desc.weights.data = _address(wts) + bind.weights_offset_bytes
+            if rows.value:
+                dev_table = task.table
+                if hasattr(src, "data_ptr"):
+                    import torch
+                    dev_table = torch.from_numpy(task.table).to(src.device)
+                task._keep.append(dev_table)
+                desc.weight_table.data = _address(dev_table)
+            task.finalize()
+            tasks.append(task)
+        return tasks
+
     def destroy(self):
         if self._handle:
             self._lib.nceHwtestDestroy(self._handle)

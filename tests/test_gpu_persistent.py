@@ -25,7 +25,8 @@ def _executor(**env):
                 os.environ[k] = v
 
 
-@pytest.mark.parametrize("batch,size", [(8, 64), (16, 96)])
+# (32, 224) is the size the benchmark times (four images per XCD: the kernel variants the full-size layers use)
+@pytest.mark.parametrize("batch,size", [(8, 64), (16, 96), (32, 224)])
 def test_resnet50_graph_persistent(batch, size):
     import torch
     executor = _executor(NCE_HIP_PERSISTENT="1")

@@ -306,3 +306,205 @@ def test_descriptors_run_bit_exact(executor, name):
     got = dout.cpu().numpy()
     assert want.std() > 1.0, "degenerate expected output"
     assert np.array_equal(got, want)
+
+
+# ---- case types that are programs of several tasks -------------------------------------------------------
+
+def program_buffers(case, rng, xp=np):
+    """Host buffers of a program: input, one weights tensor per "weight" entry, outputs in the case's output order,
+    the intermediate tensor (or None)."""
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    i = case.info.input
+    n, c, h, wd = i.shape
+    x = rng.integers(0, 256, (n, h, wd, c), dtype=np.uint8)
+    d = json.loads(case._text)
+    weights = []
+    for wl in d["weight"]:
+        oc, ic, ky, kx = wl["shape"]
+        weights.append(rng.integers(0, 256, (oc, ky, kx, ic), dtype=np.uint8))
+    outs = []
+    for s in out_shapes:
+        extent = {"n": s[0], "c": s[1], "h": s[2], "w": s[3]}
+        outs.append(np.full([extent[k] for k in case.output_order], 0x5A, dtype=np.uint8))
+    mid = np.zeros((mid_shape[0], mid_shape[2], mid_shape[3], mid_shape[1]), dtype=np.uint8) if mid_shape else None
+    return x, weights, outs, mid
+
+
+def parse_program(name, mutate=None):
+    d = json.loads(load(name))
+    if mutate:
+        mutate(d)
+    text = json.dumps(d)
+    case = hwtest.parse(text)
+    case._text = text
+    return case
+
+
+def single_conv_reference(case_json, x, wt, out_shape):
+    """The same convolution as ONE ZMajorConvolution case (no activation) on the oracle."""
+    from oracle import nce_oracle
+    d = json.loads(case_json)
+    z = {k: d[k] for k in ("architecture", "compiler_backend", "conv_op")}
+    z.update(case_type="ZMajorConvolution", input=d["input"][:1], weight=d["weight"][:1], output=[dict(d["output"][0], shape=list(out_shape))],
+             output_order="nhwc", activation={"name": None}, weights_swizzling_key=0, activation_swizzling_key=0)
+    ref_case = hwtest.parse(json.dumps(z))
+    ref = np.zeros((out_shape[0], out_shape[2], out_shape[3], out_shape[1]), dtype=np.uint8)
+    nce_oracle.run(ref_case.build_task(x, wt, ref))
+    return ref
+
+
+def nce_oracle_quant(rescale):
+    from oracle import nce_oracle
+    return nce_oracle.quant_approx(rescale)[:2]
+
+
+def run_program_on_oracle(case, x, weights, outs, mid):
+    from oracle import nce_oracle
+    tasks = case.build_program(x, weights, outs, mid)
+    for t in tasks:
+        nce_oracle.run(t)
+    return tasks
+
+
+def test_double_zmajor_convolution_is_two_chained_tasks(validator):
+    from oracle import nce_oracle
+    case = parse_program("double_zmajor_conv_u8.json")
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    assert (num_tasks, out_shapes, mid_shape, identical) == (2, [(1, 32, 16, 16)], (1, 32, 16, 16), False)
+    x, weights, outs, mid = program_buffers(case, np.random.default_rng(21))
+    tasks = run_program_on_oracle(case, x, weights, outs, mid)
+    for t in tasks:
+        validator.validate(t)
+    t0, t1 = tasks
+    assert (t0.binding.input_tensor, t0.binding.output_tensor, t0.binding.weight_layer) == (-1, -1, 0)
+    assert (t1.binding.input_tensor, t1.binding.output_tensor, t1.binding.weight_layer) == (0, 0, 1)
+    # no PPE task in this builder: NOOP with the storage range; the second convolution reads a tensor of the output's type
+    assert (t1._ppe.mode, t1._ppe.clamp_low, t1._ppe.clamp_high) == (abi.PPE_NOOP, 0, 255)
+    assert t1.desc.input.zero_point == 120 and list(t1.desc.input.dims) == [1, 32, 16, 16]
+    # both tables come from the case's input, FIRST weights and output types (hwtest.cpp:114, buildDoubleConvTest.cpp:329-360)
+    assert np.array_equal(t0.table[:, 2], t1.table[:, 2])
+    mult, shift, _ = nce_oracle.quant_approx(((0.004 + 0.0001 * 5) * 0.02) / 0.05)
+    assert t0.table[5][2] == word2(mult, shift)
+    # the chain equals two single convolutions run one after the other
+    first = single_conv_reference(case._text, x, weights[0], mid_shape)
+    assert first.std() > 1.0 and np.array_equal(mid, first)
+    d = json.loads(case._text)
+    d2 = dict(d, input=[dict(d["output"][0], shape=list(mid_shape), quantization=dict(d["output"][0]["quantization"], scale=d["input"][0]["quantization"]["scale"]))],
+              weight=[dict(d["weight"][0], shape=d["weight"][1]["shape"])])
+    second = single_conv_reference(json.dumps(d2), first, weights[1], out_shapes[0])
+    assert second.std() > 1.0 and np.array_equal(outs[0], second)
+
+
+def test_race_condition_dpu_is_the_same_task_per_cluster_and_iteration(validator):
+    case = parse_program("race_condition_dpu_u8.json")
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    assert (num_tasks, len(out_shapes), mid_shape, identical) == (6, 2, None, True)
+    x, weights, outs, mid = program_buffers(case, np.random.default_rng(22))
+    tasks = run_program_on_oracle(case, x, weights, outs, mid)
+    assert [t.binding.output_tensor for t in tasks] == [0, 1, 0, 1, 0, 1]
+    validator.validate(tasks[0])
+    ref = single_conv_reference(case._text, x, weights[0], out_shapes[0])
+    assert ref.std() > 1.0 and all(np.array_equal(o, ref) for o in outs)
+
+
+def test_different_clusters_dpu_writes_every_output_cluster(validator):
+    case = parse_program("different_clusters_dpu_u8.json")
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    assert (num_tasks, len(out_shapes), identical) == (2, 2, True)
+    x, weights, outs, mid = program_buffers(case, np.random.default_rng(23))
+    tasks = run_program_on_oracle(case, x, weights, outs, mid)
+    assert [t._variants[0].cluster_id for t in tasks] == [0, 1]
+    ref = single_conv_reference(case._text, x, weights[0], out_shapes[0])
+    assert ref.std() > 1.0 and all(np.array_equal(o, ref) for o in outs)
+    with pytest.raises(nce.NCEError) as e:
+        parse_program("different_clusters_dpu_u8.json", lambda d: d["DPUTaskParams"].pop("output_cluster"))
+    assert "loadDPUTaskParams: cannot find output_cluster config param" in e.value.log
+
+
+MULTI = [
+    ("multi_clusters_dpu_soh.json", None),
+    ("multi_clusters_dpu_soh.json", lambda d: (d["DPUTaskParams"].update(broadcast=True), d.update(output=[dict(d["output"][0], shape=[1, 32, 16, 16])] * 3))),
+    ("multi_clusters_dpu_soh.json", lambda d: d.update(output_order="nchw")),
+    ("multi_clusters_dpu_sok_broadcast.json", None),
+    ("multi_clusters_dpu_sok_broadcast.json", lambda d: (d["DPUTaskParams"].update(broadcast=False), d.update(output=[dict(d["output"][0], shape=[1, c, 9, 11]) for c in (48, 16)]))),
+]
+
+
+@pytest.mark.parametrize("name,mutate", MULTI, ids=["soh", "soh_broadcast", "soh_nchw", "sok_broadcast", "sok"])
+def test_multi_clusters_dpu_slices_make_the_whole_convolution(validator, name, mutate):
+    case = parse_program(name, mutate)
+    d = json.loads(case._text)
+    n = len(d["DPUTaskParams"]["task_clusters"])
+    broadcast = d["DPUTaskParams"]["broadcast"]
+    dim = 1 if d["DPUTaskParams"]["segmentation"] == "SOK" else 2
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    assert num_tasks == (n * n if broadcast else n) and len(out_shapes) == n and identical == broadcast
+    x, weights, outs, mid = program_buffers(case, np.random.default_rng(24))
+    tasks = run_program_on_oracle(case, x, weights, outs, mid)
+    for t in tasks:
+        validator.validate(t)
+    parent = list(out_shapes[0])
+    if not broadcast:
+        parent[dim] = sum(s[dim] for s in out_shapes)
+    ref = single_conv_reference(case._text, x, weights[0], parent)   # NHWC
+    assert ref.std() > 1.0
+    axis_of = {"n": 0, "h": 1, "w": 2, "c": 3}
+    perm = [axis_of[k] for k in case.output_order]
+    if broadcast:
+        for o in outs:
+            assert np.array_equal(o, ref.transpose(perm))
+    else:
+        start = 0
+        for o, s in zip(outs, out_shapes):
+            sl = [slice(None)] * 4
+            sl[{1: 3, 2: 1}[dim]] = slice(start, start + s[dim])
+            assert np.array_equal(o, ref[tuple(sl)].transpose(perm)), f"slice at {start}"
+            start += s[dim]
+    # SOH workloads carry the paddings of getMulticlusteringPaddings: top on the first cluster, bottom on the last
+    if dim == 2:
+        pads = [(t._variants[0].pad_top, t._variants[0].pad_bottom) for t in tasks[:n]]
+        assert pads[0] == (1, 0) and pads[-1] == (0, 1) and all(p == (0, 0) for p in pads[1:-1])
+        if not broadcast:   # each task reads only the input rows its output rows need
+            assert [int(t.desc.input.dims[2]) for t in tasks] == [7, 8, 5]
+            assert [t.binding.input_offset_bytes for t in tasks] == [0, 5 * 16 * 32, 11 * 16 * 32]
+    elif not broadcast:     # each task takes its channels' weights rows and table rows
+        assert [int(t.desc.weights.dims[0]) for t in tasks] == [48, 16] and [len(t.table) for t in tasks] == [48, 16]
+        assert [t.binding.weights_offset_bytes for t in tasks] == [0, 48 * 9 * 32]
+        assert tasks[1].table[3][2] == word2(*nce_oracle_quant((0.004 + 0.00005 * 51) * 0.02 / 0.04))
+    assert [t._variants[0].cluster_id for t in tasks[:n]] == d["DPUTaskParams"]["task_clusters"]
+
+
+PROGRAMS = ["double_zmajor_conv_u8.json", "race_condition_dpu_u8.json", "different_clusters_dpu_u8.json", "multi_clusters_dpu_soh.json",
+            "multi_clusters_dpu_sok_broadcast.json"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", PROGRAMS)
+def test_programs_run_bit_exact(executor, name):
+    """Every tensor of the program equals the oracle's; where the case says so, all outputs are byte-identical (the
+    determinism check of RaceConditionDPU: the same task, run several times into each cluster's output)."""
+    import torch
+    case = parse_program(name)
+    num_tasks, out_shapes, mid_shape, identical = case.program()
+    x, weights, outs, mid = program_buffers(case, np.random.default_rng(31))
+    run_program_on_oracle(case, x, weights, outs, mid)
+    dx = torch.from_numpy(x).cuda()
+    dws = [torch.from_numpy(w).cuda() for w in weights]
+    douts = [torch.full(o.shape, 0x5A, dtype=torch.uint8, device="cuda") for o in outs]
+    dmid = torch.zeros(mid.shape, dtype=torch.uint8, device="cuda") if mid is not None else None
+    tasks = case.build_program(dx, dws, douts, dmid, executor=executor)
+    stream = torch.cuda.current_stream().cuda_stream
+    tl = executor.task_list()
+    for t in tasks:
+        tl.append(t)
+    for rep in range(2):
+        tl.enqueue(stream)
+        executor.synchronize(stream)
+        got = [o.cpu().numpy() for o in douts]
+        for k, (g, w) in enumerate(zip(got, outs)):
+            assert w.std() > 1.0 and np.array_equal(g, w), f"run {rep} output {k}"
+        if identical:
+            assert all(np.array_equal(g, got[0]) for g in got)
+        if mid is not None:
+            assert np.array_equal(dmid.cpu().numpy(), mid)
+    tl.destroy()
