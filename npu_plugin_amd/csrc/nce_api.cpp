@@ -90,13 +90,14 @@ nce::Options read_options() {
     if (const char* e = getenv("NCE_HIP_CONV_TILE")) o.halo_tile = atoi(e);
     if (const char* e = getenv("NCE_HIP_CONV_TILED")) o.tiled = atoi(e);
     if (const char* e = getenv("NCE_HIP_CONV_PATCH")) {
-        int nf = 0, pr = 0, wv = 0;
-        const int got = sscanf(e, "%d,%d,%d", &nf, &pr, &wv);
+        int nf = 0, pr = 0, wv = 0, npx = 0;
+        const int got = sscanf(e, "%d,%d,%d,%d", &nf, &pr, &wv, &npx);
         if (got >= 2) {
             o.patch = 1;
             o.patch_nf = nf;
             o.patch_pr = pr;
-            o.patch_waves = got == 3 ? wv : 0;
+            o.patch_waves = got >= 3 ? wv : 0;
+            o.patch_npx = got >= 4 ? npx : 0;
         } else if (got == 1) {
             o.patch = nf != 0 ? 1 : 0;
         }

@@ -125,7 +125,7 @@ struct Options {
     int persistent_wait_us = 2000000;  // NCE_HIP_PERSISTENT_WAIT_US: time after which a persistent launch's waits give up
     int tiled = -1;           // NCE_HIP_CONV_TILED: -1 automatic, 0 never, 1.. force that shape of the LDS-tiled kernel
     int patch = -1;           // NCE_HIP_CONV_PATCH: -1 automatic, 0 never, 1 = wherever its conditions hold; "nf,pr[,waves]" also forces its shape
-    int patch_nf = 0, patch_pr = 0, patch_waves = 0;
+    int patch_nf = 0, patch_pr = 0, patch_waves = 0, patch_npx = 0;
     bool env_path = false;    // NCE_HIP_CONV_PATH was given at all (switches the conv + add fusion off, as NO_FUSE does)
 };
 

@@ -394,7 +394,8 @@ hipError_t launch_conv(const TaskDev& t, const Box& box, hipStream_t stream) {
     // kernel rejects.
     hipError_t e = hipErrorNotSupported;
     if (path == 0 && patch_wanted(a))
-        e = launch_conv_patch(a, stream, options().patch >= 0 ? options().patch_nf : 4, options().patch_pr, options().patch >= 0 ? options().patch_waves : 16);
+        e = launch_conv_patch(a, stream, options().patch >= 0 ? options().patch_nf : 4, options().patch_pr, options().patch >= 0 ? options().patch_waves : 16,
+                              options().patch >= 0 ? options().patch_npx : 0);
     if (e != hipErrorNotSupported) return e;
     if (const int shape = path == 0 ? tiled_shape_for(a) : 0) e = launch_conv_tiled(a, stream, shape);
     if (e != hipErrorNotSupported) return e;

@@ -227,7 +227,8 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
 // LDS-tiled kernel for many output channels; shape 1.. selects a tile shape (see nce_conv_tiled.hip), 0 the automatic choice.
 hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, const FuseAdd* fuse = nullptr);
 // Patch kernel for kernels larger than 1x1 at stride 1: weights slice and the patch's input pixels (with halo) both in LDS.
-// nf = 0 / pr = 0 / waves = 0: automatic channel fragments per slice (2 or 4) / output rows per patch / waves per workgroup (8, 16).
-hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf, int pr, int waves);
+// nf = 0 / pr = 0 / waves = 0: automatic channel fragments per slice (2 or 4) / output rows per patch / waves per workgroup (8, 16);
+// npx = 1 (with 16 waves): one pixel fragment per wave and group instead of two.
+hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf, int pr, int waves, int npx);
 
 }  // namespace nce

@@ -148,17 +148,19 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
     const int IC = a.IC;
     const int axor = (int)a.a_xor, wxor = (int)a.w_xor;
 
+    if (tid < BN) sWsum[tid] = 0;
+    __syncthreads();
+
     // ---- requests -------------------------------------------------------------------------------------------------------
+    // The last wave fetches nothing: it reads the table rows of the slice's channels (lane = channel) and derives the
+    // per-channel constants while the other waves' requests travel (a request is accepted only as fast as the memory
+    // delivers, so one wave less does not slow the transfer down).
+    constexpr int NL = NW - 1;
+    const bool consts_wave = wave == NL;
     // Weights: block wb = step * NF + fragment; lane 4 r + j fetches the piece that belongs at position j of row r.
     const int prow = lane >> 2;
     const int pj = (lane & 3) ^ swz(prow);
     const int nwblk = w.nsteps * NF;
-    for (int wb = wave; wb < nwblk; wb += NW) {
-        const int s = wb / NF, f = wb - s * NF;
-        const int ch = min(channel_of_frag_row<NF>(f, prow), noc - 1);  // rows past the box's last channel duplicate it (not stored)
-        const uint8_t* src = a.w + (int64_t)(oc0 + ch) * a.w_soc + s * 64 + pj * 16;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sL + wb * 1024), 16, 0, 0);
-    }
     // Pixels of patch pt into buffer `buf`: block k holds the slots k * (1024 / IC) ...; a lane fetches the piece that
     // belongs at its position of its slot's pixel, or the same piece of the zero-point line for a slot outside the image
     // (or beyond the patch's own rows and columns).
@@ -194,74 +196,80 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         const uint8_t* src = inside ? ps.img + (iy * in_sh32 + ix * in_sw32 + piece * 16) : fillp + (piece & 3) * 16;
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ps.dst + k * 1024), 16, 0, 0);
     };
-    auto request_patch = [&](uint32_t pt, int buf) {
+    // (first, stride): which blocks of a patch this wave fetches - and later re-biases, after its own requests have landed
+    auto request_patch = [&](uint32_t pt, int buf, int first, int stride) {
         const PatchSrc ps = patch_src(pt, buf);
-        for (int k = wave; k < w.nblk; k += NW) request_block(ps, k);
+        for (int k = first; k < w.nblk; k += stride) request_block(ps, k);
     };
-    // Re-bias, in place, the blocks of a patch buffer this wave fetched itself (after its own requests have landed).
-    auto rebias_patch = [&](int buf) {
+    auto rebias_patch = [&](int buf, int first, int stride) {
         if (axor == 0) return;  // uniform
         uint8_t* const dstb = sHalo + (uint32_t)buf * w.halo_bytes;
-        for (int k = wave; k < w.nblk; k += NW) {
+        for (int k = first; k < w.nblk; k += stride) {
             v4i* const p = reinterpret_cast<v4i*>(dstb + k * 1024 + lane * 16);
             *p = *p ^ axor;
         }
     };
-    request_patch(p_begin, 0);
-
-    if (tid < BN) sWsum[tid] = 0;
-    if (tid == 0) sFlags = 0;
-    // the table rows of the workgroup's channels travel while the operands do
-    int32_t tw2 = 0, tbias = 0;
-    if (tid < noc) {
-        const int32_t* trow = a.table + (int64_t)(oc0 + tid) * a.table_stride;
-        tw2 = trow[2];
-        tbias = trow[3];
-    }
-    __syncthreads();  // sWsum, sFlags cleared
-    PATCH_MARK(1);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    PATCH_MARK(2);
-    // weights: re-bias u8 storage; the per-channel sums of the re-biased weights when the input zero point is not the
-    // storage offset (each lane adds up the piece it fetched; the four lanes of a row combine)
-    if (wxor != 0 || a.da != 0) {
-        for (int wb = wave; wb < nwblk; wb += NW) {
-            v4i* const p = reinterpret_cast<v4i*>(sL + wb * 1024 + lane * 16);
-            v4i v = *p;
-            if (wxor != 0) {
-                v = v ^ wxor;
-                *p = v;
-            }
-            if (a.da != 0) {
-                const int f = wb % NF;
-                int32_t sum = bytesum(make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]));
-                sum += __shfl_xor(sum, 1);
-                sum += __shfl_xor(sum, 2);
-                if ((lane & 3) == 0) atomicAdd(&sWsum[channel_of_frag_row<NF>(f, prow)], sum);
-            }
-        }
-    }
-    rebias_patch(0);
-    __syncthreads();  // weights, first patch, sWsum complete
-
-    // ---- per-channel constants (thread = channel), as in the other MFMA kernels ----------------------------------------
     const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
-    if (tid < BN) {
+    if (consts_wave) {
+        int32_t tw2 = 0, tbias = 0;
+        if (lane < noc) {
+            const int32_t* trow = a.table + (int64_t)(oc0 + lane) * a.table_stride;
+            tw2 = trow[2];
+            tbias = trow[3];
+        }
         const int32_t mult = table_mult(tw2), shift = table_shift(tw2);
-        const bool bad = shift > kMaxF64Shift;
-        const bool sat = ppe_may_saturate(acc_bound, tbias, mult, shift);
+        const bool bad = lane < BN && shift > kMaxF64Shift;
+        const bool sat = lane < BN && ppe_may_saturate(acc_bound, tbias, mult, shift);
         bool hi_bad = false;
-        if (tid < noc) {
+        if (lane < noc) {
             hi_bad = shift < 1 || shift > 32 || ((int64_t)mult << (32 - min(shift, 32))) > 0x7fffffffLL;
             const double cb = ((__builtin_fabs((double)tbias) + 4294967296.0) * (double)mult + 2147483648.0 + 384.0 * __builtin_ldexp(1.0, shift));
             hi_bad = hi_bad || __builtin_ldexp(cb, 32 - shift) >= 4611686018427387904.0;
         }
-        const int wf = (bad ? 1 : 0) | (sat ? 2 : 0) | (hi_bad ? 4 : 0);
-        if (wf) atomicOr(&sFlags, wf);
-        sW2[tid] = tw2;
-        sBias[tid] = tbias;
+        const int wf = (__any(bad) ? 1 : 0) | (__any(sat) ? 2 : 0) | (__any(hi_bad) ? 4 : 0);
+        if (lane == 0) sFlags = wf;
+        if (lane < BN) {
+            const double M = ppe_scale_M(mult, shift);
+            sW2[lane] = tw2;
+            sBias[lane] = tbias;
+            sM[lane] = M;
+            sBfull[lane] = ppe_scale_B(tbias, M, shift, a.ppe.round_mode);
+        }
+    } else {
+        for (int wb = wave; wb < nwblk; wb += NL) {
+            const int s = wb / NF, f = wb - s * NF;
+            const int ch = min(channel_of_frag_row<NF>(f, prow), noc - 1);  // rows past the box's last channel duplicate it (not stored)
+            const uint8_t* src = a.w + (int64_t)(oc0 + ch) * a.w_soc + s * 64 + pj * 16;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sL + wb * 1024), 16, 0, 0);
+        }
+        request_patch(p_begin, 0, wave, NL);
+        PATCH_MARK(1);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        PATCH_MARK(2);
+        // weights: re-bias u8 storage; the per-channel sums of the re-biased weights when the input zero point is not the
+        // storage offset (each lane adds up the piece it fetched; the four lanes of a row combine)
+        if (wxor != 0 || a.da != 0) {
+            for (int wb = wave; wb < nwblk; wb += NL) {
+                v4i* const p = reinterpret_cast<v4i*>(sL + wb * 1024 + lane * 16);
+                v4i v = *p;
+                if (wxor != 0) {
+                    v = v ^ wxor;
+                    *p = v;
+                }
+                if (a.da != 0) {
+                    const int f = wb % NF;
+                    int32_t sum = bytesum(make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]));
+                    sum += __shfl_xor(sum, 1);
+                    sum += __shfl_xor(sum, 2);
+                    if ((lane & 3) == 0) atomicAdd(&sWsum[channel_of_frag_row<NF>(f, prow)], sum);
+                }
+            }
+        }
+        rebias_patch(0, wave, NL);
     }
-    __syncthreads();
+    __syncthreads();  // weights, first patch, weight sums and the constants' first part complete
+
+    // ---- per-channel constants (thread = channel), as in the other MFMA kernels ----------------------------------------
     const int flags = sFlags;
     const PpeF64 pu = ppe_f64_setup(a.ppe, (flags & 2) != 0);
     int pmode = ppe_mode_of(pu, (flags & 1) != 0);
@@ -285,12 +293,11 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
     // reference form for everything else - the FP64 forms of the other kernels would be two more copies of the epilogue.)
     if (pmode != PPE_MODE_HI && pmode != PPE_MODE_HI_SLOPE) pmode = PPE_MODE_INT;
     if (tid < BN) {
+        const int32_t tw2 = sW2[tid], tbias = sBias[tid];
         const int32_t mult = table_mult(tw2), shift = table_shift(tw2);
         const int32_t corr = a.da * sWsum[tid];  // |da| <= 255, |sum w'| < 2^23
-        const double M = ppe_scale_M(mult, shift);
-        double B = __builtin_fma((double)corr, M, ppe_scale_B(tbias, M, shift, a.ppe.round_mode));
+        double B = __builtin_fma((double)corr, sM[tid], sBfull[tid]);
         if (pmode != PPE_MODE_INT) B += ep.zp_fold;  // floor(x + zp) = floor(x) + zp
-        sM[tid] = M;
         sBfull[tid] = B;
         sCorr[tid] = corr;
         if (pmode == PPE_MODE_HI || pmode == PPE_MODE_HI_SLOPE) {
@@ -347,7 +354,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         auto finish_next = [&]() {
             for (; kreq < w.nblk; kreq += NW) request_block(nx, kreq);  // (what the reduction steps did not get to)
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            rebias_patch(buf ^ 1);
+            rebias_patch(buf ^ 1, wave, NW);
             next_done = true;
         };
         PATCH_MARK_SEQ();   // patch top (after the next patch's requests)
@@ -409,8 +416,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
                     kreq += NW;
                 }
             };
-            if constexpr (NW == 8) {
-                // Two waves per SIMD: two register sets, so that the reads of step s + 1 are in flight while the matrix
+            if constexpr (NW == 8 || NF == 2) {
+                // Two waves per SIMD (or registers to spare): two register sets, so that the reads of step s + 1 are in flight while the matrix
                 // instructions of step s run. (Both requests of the loop body are unconditional and the tail is written out,
                 // so that every block of matrix instructions follows the requests of the step after it on every path: the
                 // wait before it then names just the older set, and the younger one stays in flight.)
@@ -477,9 +484,9 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         if (more) {
             if (w.nbuf == 1) {
                 __syncthreads();  // every wave has left the only buffer
-                request_patch(pt + 1, 0);
+                request_patch(pt + 1, 0, wave, NW);
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-                rebias_patch(0);
+                rebias_patch(0, wave, NW);
                 __syncthreads();
             } else {
                 if (!next_done) finish_next();  // (a wave without a group in this patch)
@@ -505,7 +512,15 @@ hipError_t launch_patch(const PatchArgs& w, size_t lds, hipStream_t stream) {
 }
 
 template <int NF>
-hipError_t launch_patch_u(const PatchArgs& w, size_t lds, int ulog, int waves, hipStream_t stream) {
+hipError_t launch_patch_u(const PatchArgs& w, size_t lds, int ulog, int waves, int npxf, hipStream_t stream) {
+    if (waves == 16 && npxf == 1) {
+        switch (ulog) {
+        case 2: return launch_patch<NF, 1, 2, 16>(w, lds, stream);
+        case 3: return launch_patch<NF, 1, 3, 16>(w, lds, stream);
+        case 4: return launch_patch<NF, 1, 4, 16>(w, lds, stream);
+        default: return hipErrorNotSupported;
+        }
+    }
     if (waves == 16) {
         switch (ulog) {
         case 2: return launch_patch<NF, 2, 2, 16>(w, lds, stream);
@@ -525,10 +540,11 @@ hipError_t launch_patch_u(const PatchArgs& w, size_t lds, int ulog, int waves, h
 }  // namespace
 
 // nf_forced: 0 = automatic, 2 or 4 = channel fragments per slice; pr_forced: 0 = automatic, else output rows per patch;
-// waves_forced: 0 = automatic, 8 or 16 = waves per workgroup (groups of four or two pixel fragments).
-hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_forced, int pr_forced, int waves_forced) {
+// waves_forced: 0 = automatic, 8 or 16 = waves per workgroup (groups of four or two pixel fragments); npx_forced = 1 with 16
+// waves: groups of one pixel fragment (small patches: a group per wave).
+hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_forced, int pr_forced, int waves_forced, int npx_forced) {
     const int waves = waves_forced == 16 ? 16 : 8;
-    const int npxf = waves == 16 ? 2 : 4;  // pixel fragments per group
+    const int npxf = waves == 16 ? (npx_forced == 1 ? 1 : 2) : 4;  // pixel fragments per group
     if (a.SY != 1 || a.SX != 1 || a.dw != 0) return hipErrorNotSupported;
     if (a.IC != 64 && a.IC != 128 && a.IC != 256 && a.IC != 512 && a.IC != 1024) return hipErrorNotSupported;
     if (a.KY > 16 || a.KX > 16 || a.bw > 4096 || a.bh > 32768) return hipErrorNotSupported;
@@ -611,10 +627,10 @@ hipError_t launch_conv_patch(const ConvArgs& a, hipStream_t stream, int nf_force
     w.trace = g_probe_trace;
 #endif
     if (tls_launch.log != nullptr)
-        tls_launch.log->add(3, "conv: patch kernel, %d channels per slice, %d rows per patch, %d patch buffer(s), %u workgroups of %d waves x %u patches",
-                            16 * nf, w.PR, w.nbuf, w.ngroups * w.nslices, waves, w.tpg);
-    if (nf == 4) return launch_patch_u<4>(w, lds, ulog, waves, stream);
-    return launch_patch_u<2>(w, lds, ulog, waves, stream);
+        tls_launch.log->add(3, "conv: patch kernel, %d channels per slice, %d rows per patch, %d patch buffer(s), %u workgroups of %d waves x %u patches, groups of %d fragment(s)",
+                            16 * nf, w.PR, w.nbuf, w.ngroups * w.nslices, waves, w.tpg, npxf);
+    if (nf == 4) return launch_patch_u<4>(w, lds, ulog, waves, npxf, stream);
+    return launch_patch_u<2>(w, lds, ulog, waves, npxf, stream);
 }
 
 }  // namespace nce

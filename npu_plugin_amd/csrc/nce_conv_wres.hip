@@ -22,12 +22,14 @@
 // 64 a step never straddles taps and the tap bookkeeping is scalar; other channel counts take the
 // per-lane path (template MODE 2). Semantics and the fused PPE are the ones of nce_conv.hip.
 #include "nce_conv_epi.h"
+#include "nce_conv_lds.h"
 #include "nce_conv_pk.h"
 
 #include <mutex>
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 namespace nce {
 
@@ -51,7 +53,20 @@ struct WresArgs {
     int32_t in_sn32, in_sh32, in_sw32, out_sn32, out_sh32, out_sw32;
     FuseAdd fz;         // kernels with LM_PLAIN_FZ only
     int32_t fused;      // host: the launch must carry the add in fz (or fail with hipErrorNotSupported)
+#ifdef WRES_TRACE
+    uint64_t* trace;    // probe builds only: [workgroup < 256][wave < 8][8] timestamps (100 MHz) of this launch
+#endif
 };
+
+#ifdef WRES_TRACE
+#define WRES_MARK(i)                                                                                                       \
+    do {                                                                                                                   \
+        if (w.trace != nullptr && lane == 0 && blockIdx.x < 256)                                                           \
+            w.trace[((size_t)blockIdx.x * 8 + wave) * 8 + (i)] = __builtin_amdgcn_s_memrealtime();                          \
+    } while (0)
+#else
+#define WRES_MARK(i) do { } while (0)
+#endif
 
 // This file is compiled four times (the instantiations of one pass take about a minute): WRES_PART 0 holds the dispatcher,
 // the 32-channel kernels and the chunked kernel, WRES_PART 1 the 64-channel kernels with 16- and 32-pixel tiles behind this
@@ -60,6 +75,10 @@ struct WresArgs {
 #define WRES_PART 0
 #endif
 hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream);
+#ifdef WRES_TRACE
+extern uint64_t* g_wres_trace;  // probe builds: 64 launch records, written round robin
+extern uint32_t g_wres_trace_seq;
+#endif
 
 namespace {
 
@@ -130,7 +149,6 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
     constexpr bool FZ = LM == LM_PLAIN_FZ;
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
-    constexpr int WB = 4;      // weight loads in flight per lane while staging
     static_assert(NF == 2 || NF == 4, "channel fragments");
     static_assert(D >= 2 || !TRL, "the permute of the next step needs a second ring slot");
     static_assert(!(TRL && TBL) && !(TBL && MODE == WRES_GENERIC), "the step table serves the plain load order of modes 0 and 1");
@@ -325,7 +343,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
     // lanes), permutes the registers into operand order (lane 16k + i) and writes the fragment with one
     // linear, bank-conflict-free store.
     {
-        const int li = lane >> 2, lk = kswz;
+        const int li = lane >> 2;
         const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
         // The last wave also derives the per-channel PPE constants (lane = channel) while its weight
         // loads are in flight.
@@ -360,12 +378,17 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
                 sBc[lane] = B;
             }
         };
-        // Row (channel) this lane fetches in each channel fragment.
+        // Reduction step st, channel fragment f is one 1 KiB block of 16 rows (channels) x 64 bytes, kept row-major: lane
+        // 4 r + j fetches the 16-byte piece that belongs at position j of row r (nce_conv_lds.h: the pieces of a row are
+        // permuted so that the operand reads of the reduction loop touch every bank group once per clock), and writes it
+        // where it stands - one linear, conflict-free store per block. Rows past the slice's last channel and pieces past
+        // the reduction's end are zero.
+        const int pj = (lane & 3) ^ lds_detail::swz(li);
         const uint8_t* wrow[NF];
         bool wrow_ok[NF];
         // (fragment f's row is 4 * f below fragment 0's: one 64-bit multiply, then uniform additions; rows past the
         // slice's last channel are never dereferenced)
-        const uint8_t* const wrow0 = a.w + (int64_t)(oc0 + channel_of_frag_row<NF>(0, li)) * a.w_soc + lk * 16;
+        const uint8_t* const wrow0 = a.w + (int64_t)(oc0 + channel_of_frag_row<NF>(0, li)) * a.w_soc + pj * 16;
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
             wrow_ok[f] = channel_of_frag_row<NF>(f, li) < noc;
@@ -374,6 +397,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         int32_t wpart[NF];  // sum of the (signed) weights this lane staged, per channel fragment
 #pragma unroll
         for (int f = 0; f < NF; ++f) wpart[f] = 0;
+        constexpr int WB = 4;       // weight loads in flight per lane while staging
         constexpr int SB = WB / NF;  // steps per batch of loads
         uint4 v[SB][NF];
         // requests only (nothing here consumes a loaded value) ...
@@ -381,7 +405,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
 #pragma unroll
             for (int j = 0; j < SB; ++j) {
                 const int st = s0 + j * nwaves;
-                const bool in_k = st < S && 4 * st + lk < w.k16;
+                const bool in_k = st < S && 4 * st + pj < w.k16;
 #pragma unroll
                 for (int f = 0; f < NF; ++f) {
                     // (padding holds the XOR mask itself, so that the unconditional XOR below turns it into zero;
@@ -391,7 +415,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
                 }
             }
         };
-        // ... then the weight sums, permutes and LDS writes
+        // ... then the weight sums and LDS writes
         auto commit = [&](int s0) {
 #pragma unroll
             for (int j = 0; j < SB; ++j) {
@@ -400,16 +424,8 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
 #pragma unroll
                     for (int f = 0; f < NF; ++f) {
                         const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
-                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.x, 0x01010101, wpart[f], false);
-                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.y, 0x01010101, wpart[f], false);
-                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.z, 0x01010101, wpart[f], false);
-                        wpart[f] = __builtin_amdgcn_sdot4((int)sw.w, 0x01010101, wpart[f], false);
-                        uint4 x;
-                        x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.x);
-                        x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.y);
-                        x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.z);
-                        x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.w);
-                        *reinterpret_cast<uint4*>(sWt + ((size_t)st * NF + f) * 1024 + lane * 16) = x;
+                        wpart[f] += bytesum(sw);
+                        *reinterpret_cast<uint4*>(sWt + ((size_t)st * NF + f) * 1024 + lane * 16) = sw;
                     }
                 }
             }
@@ -418,10 +434,12 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         // first activation requests and the constants run while they are in flight.
         // (No branch around these activation requests - the wait for the weights would otherwise have to cover
         // them too; a wave without a tile requests the last pixel's data, which setup() clamps to.)
+        WRES_MARK(0);
         request(wave);
         input_wait();
         setup();
         first_loads(false);
+        WRES_MARK(1);
         if (consts_wave) do_consts();
         commit(wave);
         for (int s0 = wave + nwaves * SB; s0 < S; s0 += nwaves * SB) {
@@ -434,7 +452,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
             int32_t p = wpart[f];
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
-            if (lk == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
+            if ((lane & 3) == 0) sWpart[wave][channel_of_frag_row<NF>(f, li)] = p;
         }
     }
     if constexpr (TBL) {
@@ -442,7 +460,9 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
     } else if (MODE == WRES_GENERIC) {
         for (int u = tid; u < 4 * S; u += (int)blockDim.x) sStep[u] = unit_entry(u);
     }
+    WRES_MARK(2);
     __syncthreads();  // weights and constants are in LDS; no workgroup synchronisation after this
+    WRES_MARK(3);
 
     const int flags = sFlags;
     const PpeF64 pu = ppe_f64_setup(ppe_args, (flags & 2) != 0);
@@ -494,7 +514,10 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
     }
     // (same wave writes and reads: program order is enough, the compiler waits on the LDS counter)
 
+    // weights: lane (c16, q) reads piece q of row c16 of a block
+    const int wfrag_off = c16 * 64 + (((lane >> 4) ^ lds_detail::swz(c16)) << 4);
     // ---- per-wave tile loop -----------------------------------------------------------------------
+    WRES_MARK(4);
     while (t < t_end) {
         v4i acc[NF][BF];
 #pragma unroll
@@ -516,7 +539,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
 #pragma unroll
         for (int x = 0; x < BF; ++x) asum[x] = v4i{0, 0, 0, 0};
         const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-        const uint8_t* ap = sWt + lane * 16;
+        const uint8_t* ap = sWt + wfrag_off;
         v4i fa[NF];
 #pragma unroll
         for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
@@ -583,6 +606,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         int32_t dws[BF];  // every row of asum holds the pixel's sum: register 0 of this lane is its column's
 #pragma unroll
         for (int x = 0; x < BF; ++x) dws[x] = ASUM ? a.dw * asum[x][0] : 0;
+        WRES_MARK(5);  // (of the wave's last tile)
         if (pmode == PPE_MODE_HI) wres_epilogue<NF, BF, PPE_MODE_HI, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
         else if (pmode == PPE_MODE_HI_SLOPE) wres_epilogue<NF, BF, PPE_MODE_HI_SLOPE, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
         else if (pmode == PPE_MODE_FOLDED) wres_epilogue<NF, BF, PPE_MODE_FOLDED, FZ>(a, es, sBfull[wave], sCorr[wave], acc, dws, lane >> 4, noc, dst, valid, pu, ep, &w.fz, other);
@@ -594,6 +618,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
             first_loads(true);
         }
     }
+    WRES_MARK(6);
 }
 
 template <int NF, int BF, int MODE, int D, int LM>
@@ -1046,11 +1071,22 @@ hipError_t launch_wres_nf4_bf4(WresArgs& w, int mode, int nwaves, int tpw, hipSt
     return launch_mode<4, 4>(w, mode, nwaves, tpw, stream);
 }
 #elif WRES_PART == 0
+#ifdef WRES_TRACE
+uint64_t* g_wres_trace = nullptr;
+uint32_t g_wres_trace_seq = 0;
+extern "C" void nceProbeSetWresTrace(uint64_t* device_buffer) {
+    g_wres_trace = device_buffer;
+    g_wres_trace_seq = 0;
+}
+#endif
 hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_chunked, const FuseAdd* fuse) {
     if (a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     // (pixel indices of tiles past the end - waves without a tile still form addresses - must stay below 2^31)
     if (a.M > 0x7fffffff - 64 * 1024) return hipErrorNotSupported;
     WresArgs w;
+#ifdef WRES_TRACE
+    w.trace = g_wres_trace != nullptr ? g_wres_trace + (size_t)(g_wres_trace_seq++ % 64) * 256 * 8 * 8 : nullptr;
+#endif
     w.a = a;
     w.fused = fuse != nullptr;
     if (fuse) w.fz = *fuse;
