@@ -823,7 +823,7 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
     };
 
     // ---- weight staging (see conv_wres_kernel) ---------------------------------------------------------------
-    const int li = lane >> 2, lk = lane & 3;
+    const int li = lane >> 2, lk = (lane & 3) ^ lds_detail::swz(li);  // row and piece this lane stages (blocks stay row-major)
     const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
     const bool consts_wave = wave == nwaves - 1;
     int32_t tw2 = 0, tbias = 0;
@@ -865,16 +865,8 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
 #pragma unroll
                 for (int f = 0; f < NF; ++f) {
                     const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
-                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.x, 0x01010101, wpart[f], false);
-                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.y, 0x01010101, wpart[f], false);
-                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.z, 0x01010101, wpart[f], false);
-                    wpart[f] = __builtin_amdgcn_sdot4((int)sw.w, 0x01010101, wpart[f], false);
-                    uint4 x;
-                    x.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.x);
-                    x.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.y);
-                    x.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.z);
-                    x.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_mfma, (int)sw.w);
-                    *reinterpret_cast<uint4*>(sWt + ((size_t)(st - sbase) * NF + f) * 1024 + lane * 16) = x;
+                    wpart[f] += bytesum(sw);
+                    *reinterpret_cast<uint4*>(sWt + ((size_t)(st - sbase) * NF + f) * 1024 + lane * 16) = sw;
                 }
             }
         }
@@ -943,7 +935,7 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
             }
         }
         __syncthreads();  // the chunk is in LDS
-        const uint8_t* ap = sWt + lane * 16;
+        const uint8_t* ap = sWt + (lane & 15) * 64 + (((lane >> 4) ^ lds_detail::swz(lane & 15)) << 4);  // piece lane / 16 of row lane % 16
         v4i fa[NF];
 #pragma unroll
         for (int f = 0; f < NF; ++f) fa[f] = *reinterpret_cast<const v4i*>(ap + f * 1024);
