@@ -33,5 +33,16 @@ constexpr int vmcnt_imm(int n) {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
+// One global_load_lds_dwordx4: lane l's 16 bytes at `src` go to LDS at `block` + 16 l (block: uniform, a pointer into
+// __shared__ memory). Written as inline assembly on purpose: in a kernel that contains the compiler's own builtin for
+// this instruction, every wait the compiler inserts on the LDS counter is a wait for ALL outstanding LDS reads (it no
+// longer counts them), which serialises each ds_read with its use; the assembly form leaves its counting intact. The
+// transfer counts as a vector-memory operation: wait with vmcnt (vmcnt_imm) - and a barrier, for other waves - before the
+// block is read. The "memory" clobber keeps the compiler from moving LDS or global accesses across the request.
+__device__ __forceinline__ void load_to_lds_16(const void* src, void* block) {
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)block;
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+}
+
 }  // namespace lds_detail
 }  // namespace nce

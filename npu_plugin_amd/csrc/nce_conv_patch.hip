@@ -34,6 +34,7 @@
 #include "nce_conv_lds.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         const int piece = halo_piece<ULOG>(iy * a.bw + ix, lane_pos);
         const bool inside = (uint32_t)(iy - ps.iy_lo) < (uint32_t)ps.iy_n && (uint32_t)(ix - ps.ix_lo) < (uint32_t)ps.ix_n;
         const uint8_t* src = inside ? ps.img + (iy * in_sh32 + ix * in_sw32 + piece * 16) : fillp + (piece & 3) * 16;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ps.dst + k * 1024), 16, 0, 0);
+        load_to_lds_16(src, ps.dst + k * 1024);
     };
     // (first, stride): which blocks of a patch this wave fetches - and later re-biases, after its own requests have landed
     auto request_patch = [&](uint32_t pt, int buf, int first, int stride) {
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
             const int s = wb / NF, f = wb - s * NF;
             const int ch = min(channel_of_frag_row<NF>(f, prow), noc - 1);  // rows past the box's last channel duplicate it (not stored)
             const uint8_t* src = a.w + (int64_t)(oc0 + ch) * a.w_soc + s * 64 + pj * 16;
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sL + wb * 1024), 16, 0, 0);
+            load_to_lds_16(src, sL + wb * 1024);
         }
         request_patch(p_begin, 0, wave, NL);
         PATCH_MARK(1);
@@ -339,7 +340,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         const bool ahead = w.nbuf == 2 && more;
         PatchSrc nx = {};
         if (ahead) nx = patch_src(pt + 1, buf ^ 1);
-        int kreq = ahead ? wave : w.nblk;  // this wave's next block to request
+        const int req_first = wave, req_stride = NW;  // this wave's blocks of the next patch
+        int kreq = ahead ? req_first : w.nblk;  // this wave's next block to request
         const uint8_t* const hb = sHalo + (uint32_t)buf * w.halo_bytes;
         const int32_t n = (int32_t)fdiv(pt, w.div_nrp);
         const int32_t row0 = ((int32_t)pt - n * w.nrp) * w.PR;
@@ -352,9 +354,9 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
         // (long landed) and not the stores that epilogue is about to issue.
         bool next_done = !ahead;
         auto finish_next = [&]() {
-            for (; kreq < w.nblk; kreq += NW) request_block(nx, kreq);  // (what the reduction steps did not get to)
+            for (; kreq < w.nblk; kreq += req_stride) request_block(nx, kreq);  // (what the reduction steps did not get to)
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            rebias_patch(buf ^ 1, wave, NW);
+            rebias_patch(buf ^ 1, req_first, req_stride);
             next_done = true;
         };
         PATCH_MARK_SEQ();   // patch top (after the next patch's requests)
@@ -386,17 +388,15 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
 #pragma unroll
                 for (int x = 0; x < NPX; ++x) fb[x] = *reinterpret_cast<const v4i*>(hb + (abase[x] + tapoff + ((akq[x] + ts) & POSMASK)));
                 wp += NF * 1024;
-#ifdef PATCH_KO_WALK
-                if (false) {
-#else
-                if (++it_c == w.nc64) {
-#endif
-                    it_c = 0;
-                    if (++it_kx == a.KX) {
-                        it_kx = 0;
-                        ++it_ky;
-                    }
-                }
+                // (selects, no branches: between the reads of one step and the matrix instructions of the other the code
+                // must stay one block, or the wait before those instructions also covers the reads just issued)
+                ++it_c;
+                const bool wrap_c = it_c == w.nc64;
+                it_c = wrap_c ? 0 : it_c;
+                it_kx += wrap_c ? 1 : 0;
+                const bool wrap_x = it_kx == a.KX;
+                it_kx = wrap_x ? 0 : it_kx;
+                it_ky += wrap_x ? 1 : 0;
             };
             auto mma = [&](const v4i (&fa)[NF], const v4i (&fb)[NPX]) {
 #pragma unroll
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
                 if (kreq < w.nblk) {  // uniform
 #endif
                     request_block(nx, kreq);
-                    kreq += NW;
+                    kreq += req_stride;
                 }
             };
             if constexpr (NW == 8 || NF == 2) {
@@ -422,20 +422,35 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
                 // so that every block of matrix instructions follows the requests of the step after it on every path: the
                 // wait before it then names just the older set, and the younger one stays in flight.)
                 v4i fa0[NF], fb0[NPX], fa1[NF], fb1[NPX];
+                // (Nothing but LDS reads may be outstanding on the LDS counter inside the loop: with a scalar load still
+                // counted there - they return out of order - every wait in the loop would be a wait for everything.)
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+                constexpr int kWaitOlderSet = 0xC07F | ((NF + NPX) << 8);  // lgkmcnt(NF + NPX): all but the reads of the newest step
                 fetch(fa0, fb0);
-                if (Sn > 1) fetch(fa1, fb1);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(fa1, fb1);  // (unconditional, like every fetch here: a reduction of one step reads, and ignores, what follows)
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(kWaitOlderSet);
 #pragma unroll
                 for (int f = 0; f < NF; ++f)  // the first step starts the accumulators (no zeroing pass)
 #pragma unroll
                     for (int x = 0; x < NPX; ++x) acc[f][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa0[f], fb0[x], zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
                 int s = 1;
                 for (; s + 2 < Sn; s += 2) {
+                    // (the fences keep the compiler from sinking a step's reads to just above their use)
                     fetch(fa0, fb0);
                     request_one();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_waitcnt(kWaitOlderSet);
                     mma(fa1, fb1);
+                    __builtin_amdgcn_sched_barrier(0);
                     fetch(fa1, fb1);
                     request_one();
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_waitcnt(kWaitOlderSet);
                     mma(fa0, fb0);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 if (s + 1 < Sn) {
                     fetch(fa0, fb0);

@@ -135,12 +135,12 @@ __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_t
             uint8_t* const st = sT + slot * STAGE + c * CHUNK + wave * 1024;
 #pragma unroll
             for (int i = 0; i < NA; ++i)
-                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + w_off + 64 * c), (lptr_t)(st + NW * i * 1024), 16, 0, 0);
+                load_to_lds_16(wsrc[i] + w_off + 64 * c, st + NW * i * 1024);
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 const uint8_t* src = bsrc[i] + it_off + 64 * c;
                 if (!w.inside) src = ((rows[i] >> it_ky) & (cols[i] >> it_kx) & 1u) ? src : fillp;
-                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + (ABLK + NW * i) * 1024), 16, 0, 0);
+                load_to_lds_16(src, st + (ABLK + NW * i) * 1024);
             }
         }
         w_off += 64 * KC;
