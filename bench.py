@@ -112,7 +112,7 @@ def make_scaled_workloads():
 MIN_WARM_S = 0.03  # every measurement is preceded by at least this much GPU work (clocks ramp on an idle device)
 
 
-STEPS_RUN = [0]  # steps of the main workload enqueued so far, warm-up included (what --marks reports)
+STEPS_RUN = [0]  # steps enqueued so far, warm-up and timed (--marks reports the count after the main workload)
 
 
 def warm_up(run, count, per_run=1):
@@ -131,8 +131,10 @@ def warm_up(run, count, per_run=1):
     return done
 
 
-def time_task(ex, dc, steps, warmup):
-    """Returns (wall seconds per step, event seconds per step)."""
+def time_task(ex, dc, steps, warmup, reps=1):
+    """Returns (wall seconds per step, event seconds per step); with reps > 1 the median of that many timed runs of
+    `steps` steps each (the side workloads: 3-15 us per step, where one run's figure moves by several per cent with the
+    launch jitter of the moment)."""
     import torch
     stream = torch.cuda.current_stream().cuda_stream
     warm = ex.task_list()
@@ -142,24 +144,29 @@ def time_task(ex, dc, steps, warmup):
     for _ in range(steps):
         timed.append(dc.task)
     warm_up(lambda: warm.enqueue(stream), 1, per_run=max(warmup, 1))
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    timed.enqueue(stream)
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    runs = []
+    for _ in range(max(1, reps)):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        timed.enqueue(stream)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        STEPS_RUN[0] += steps
+        runs.append(((t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps))
     warm.destroy()
     timed.destroy()
-    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+    runs.sort(key=lambda r: r[1])
+    return runs[len(runs) // 2]
 
 
-def measure(ex, name, maker, bound, steps, warmup):
+def measure(ex, name, maker, bound, steps, warmup, reps=1):
     from npu_plugin_amd import workloads as W
     case = maker()
     dc = W.DeviceCase(case)
-    wall, ev = time_task(ex, dc, steps, warmup)
+    wall, ev = time_task(ex, dc, steps, warmup, reps)
     ops, nbytes = case.ops(), case.algorithmic_bytes()
     if bound == "mfma":
         value, unit = ops / wall / 1e9, "GOPS"
@@ -219,6 +226,7 @@ def measure_graph(ex, steps, warmup, batch=32, per_layer=False):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     ev = e0.elapsed_time(e1) * 1e-3 / steps
+    STEPS_RUN[0] += steps
     ops = graph.conv_ops()
     conv_bytes = sum(graph.layer_bytes(L) for L in graph.layers if L.task_type == 0)
     other_bytes = sum(graph.layer_bytes(L) for L in graph.layers if L.task_type != 0)
@@ -305,6 +313,7 @@ def measure_chain(ex, steps, warmup):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     ev = e0.elapsed_time(e1) * 1e-3 / steps
+    STEPS_RUN[0] += steps
     warm.destroy()
     timed.destroy()
     # algorithmic bytes of the chain: input and weights once, every output once (the intermediates are outputs of the
@@ -327,6 +336,7 @@ def main():
     ap.add_argument("--no-others", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-scaled", action="store_true", help="skip the large-batch variants of the workloads")
+    ap.add_argument("--batch", type=int, default=32, help="cfg5 only: batch of the graph (profiling; the headline is 32)")
     ap.add_argument("--per-layer", action="store_true", help="cfg5: print a per-task timing table on stderr")
     ap.add_argument("--traffic-reference", action="store_true",
                     help="also run plain 256 MiB device copies, the known-size reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
@@ -363,21 +373,21 @@ def main():
     side_steps = max(args.steps, 200)
     if args.workload == "cfg5":
         case, bound = None, "mfma"
-        main_res = measure_graph(ex, graph_steps, graph_warm, per_layer=args.per_layer)
+        main_res = measure_graph(ex, graph_steps, graph_warm, batch=args.batch, per_layer=args.per_layer)
         main_res["bytes_per_step"] = main_res["conv_bytes_per_step"] + main_res["pool_add_bytes_per_step"]
         workload_name = main_res["workload"]
-        steps_total = graph_steps + graph_warm
+        steps_total = STEPS_RUN[0]
     elif args.workload == "cfg3_chain":
         case, bound = None, "hbm"
         main_res = measure_chain(ex, args.steps, args.warmup)
         main_res["ops_per_step"] = 0
         workload_name = main_res["workload"]
-        steps_total = args.steps + max(1, args.warmup)
+        steps_total = STEPS_RUN[0]
     else:
         maker, bound = workloads[args.workload]
         case, main_res = measure(ex, args.workload, maker, bound, args.steps, args.warmup)
         workload_name = case.name
-        steps_total = args.steps + max(1, args.warmup)
+        steps_total = STEPS_RUN[0]
     if args.marks:
         with open(args.marks, "w") as f:
             json.dump({"workload": args.workload, "steps_total": steps_total, "algorithmic_bytes": main_res["bytes_per_step"]}, f)
@@ -402,7 +412,7 @@ def main():
         for name, (mk, bd) in workloads.items():
             if name == args.workload:
                 continue
-            _, r = measure(ex, name, mk, bd, side_steps, args.warmup)
+            _, r = measure(ex, name, mk, bd, side_steps, args.warmup, reps=5)
             others[name] = r
         if args.workload != "cfg3_chain":
             others["cfg3_chain"] = measure_chain(ex, side_steps, args.warmup)
