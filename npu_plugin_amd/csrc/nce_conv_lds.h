@@ -41,7 +41,12 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // block is read. The "memory" clobber keeps the compiler from moving LDS or global accesses across the request.
 __device__ __forceinline__ void load_to_lds_16(const void* src, void* block) {
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)block;
+    // (m0 is named as clobbered so that the compiler does not carry a value of its own in it across the request; it warns
+    // about reserved registers in clobber lists in general)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+#pragma clang diagnostic pop
 }
 
 }  // namespace lds_detail

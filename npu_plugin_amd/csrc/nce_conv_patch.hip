@@ -204,9 +204,22 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w
     };
     auto rebias_patch = [&](int buf, int first, int stride) {
         if (axor == 0) return;  // uniform
-        uint8_t* const dstb = sHalo + (uint32_t)buf * w.halo_bytes;
-        for (int k = first; k < w.nblk; k += stride) {
-            v4i* const p = reinterpret_cast<v4i*>(dstb + k * 1024 + lane * 16);
+        uint8_t* const dstb = sHalo + (uint32_t)buf * w.halo_bytes + lane * 16;
+        // four blocks at a time: read, XOR and write back one by one, a wave pays one LDS round trip per block
+        int k = first;
+        for (; k + 3 * stride < w.nblk; k += 4 * stride) {
+            v4i* const p0 = reinterpret_cast<v4i*>(dstb + k * 1024);
+            v4i* const p1 = reinterpret_cast<v4i*>(dstb + (k + stride) * 1024);
+            v4i* const p2 = reinterpret_cast<v4i*>(dstb + (k + 2 * stride) * 1024);
+            v4i* const p3 = reinterpret_cast<v4i*>(dstb + (k + 3 * stride) * 1024);
+            const v4i v0 = *p0, v1 = *p1, v2 = *p2, v3 = *p3;
+            *p0 = v0 ^ axor;
+            *p1 = v1 ^ axor;
+            *p2 = v2 ^ axor;
+            *p3 = v3 ^ axor;
+        }
+        for (; k < w.nblk; k += stride) {
+            v4i* const p = reinterpret_cast<v4i*>(dstb + k * 1024);
             *p = *p ^ axor;
         }
     };

@@ -36,7 +36,7 @@ def _id(s):
     return f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}x{s[5][1]}"
 
 
-@pytest.mark.parametrize("knob", ["1", "4,1", "4,3", "2,5", "2,64", "4,3,16", "2,6,16"])
+@pytest.mark.parametrize("knob", ["1", "4,1", "4,3", "2,5", "2,64", "4,3,16", "2,6,16", "2,14,16,1"])
 @pytest.mark.parametrize("shape", PATCH_SHAPES, ids=_id)
 def test_conv_patch_shapes(tuned, shape, knob):
     n, h, w, ic, oc, k, pads, in_zp = shape
