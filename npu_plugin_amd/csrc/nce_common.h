@@ -66,6 +66,50 @@ __device__ inline uint32_t xcd_tile(uint32_t block_id, uint32_t ntiles) {
     return (block_id % kNumXcd) * per_xcd + block_id / kNumXcd;
 }
 
+// Kernel arguments sit in memory and reach the scalar registers through scalar loads that the compiler places next to
+// their first use: a kernel with a few hundred bytes of arguments then starts with a CHAIN of cold misses, one per group
+// of 64-byte lines it touches for the first time (four in the weights-resident convolution: 0.3-0.7 us each from memory,
+// with a wait between them). Called first thing in a kernel, this requests one word of every line of the argument block
+// at once and waits for them together; the compiler's own loads then find the lines in the scalar cache.
+// BYTES = sizeof of the kernel's argument struct (its only parameter).
+template <int BYTES>
+__device__ __forceinline__ void prefetch_kernel_arguments() {
+#ifdef __HIP_DEVICE_COMPILE__
+    constexpr int LINES = (BYTES + 63) / 64;
+    static_assert(LINES >= 1 && LINES <= 16, "argument block larger than this helper covers");
+    const auto p = __builtin_amdgcn_kernarg_segment_ptr();  // (constant address space)
+    // (one statement: the loaded words are thrown away, and a register the compiler took back before the word arrived
+    // would be overwritten later)
+    int t[16];
+#define NCE_KA_LOAD(i) "s_load_dword %" #i ", %16, " #i "*64\n\t"
+    if constexpr (LINES <= 4) {
+        asm volatile(NCE_KA_LOAD(0) NCE_KA_LOAD(1) NCE_KA_LOAD(2) NCE_KA_LOAD(3) "s_waitcnt lgkmcnt(0)"
+                     : "=s"(t[0]), "=s"(t[1]), "=s"(t[2]), "=s"(t[3]), "=s"(t[4]), "=s"(t[5]), "=s"(t[6]), "=s"(t[7]), "=s"(t[8]), "=s"(t[9]), "=s"(t[10]),
+                       "=s"(t[11]), "=s"(t[12]), "=s"(t[13]), "=s"(t[14]), "=s"(t[15])
+                     : "s"(p));
+    } else if constexpr (LINES <= 8) {
+        asm volatile(NCE_KA_LOAD(0) NCE_KA_LOAD(1) NCE_KA_LOAD(2) NCE_KA_LOAD(3) NCE_KA_LOAD(4) NCE_KA_LOAD(5) NCE_KA_LOAD(6) NCE_KA_LOAD(7) "s_waitcnt lgkmcnt(0)"
+                     : "=s"(t[0]), "=s"(t[1]), "=s"(t[2]), "=s"(t[3]), "=s"(t[4]), "=s"(t[5]), "=s"(t[6]), "=s"(t[7]), "=s"(t[8]), "=s"(t[9]), "=s"(t[10]),
+                       "=s"(t[11]), "=s"(t[12]), "=s"(t[13]), "=s"(t[14]), "=s"(t[15])
+                     : "s"(p));
+    } else if constexpr (LINES <= 12) {
+        asm volatile(NCE_KA_LOAD(0) NCE_KA_LOAD(1) NCE_KA_LOAD(2) NCE_KA_LOAD(3) NCE_KA_LOAD(4) NCE_KA_LOAD(5) NCE_KA_LOAD(6) NCE_KA_LOAD(7) NCE_KA_LOAD(8)
+                     NCE_KA_LOAD(9) NCE_KA_LOAD(10) NCE_KA_LOAD(11) "s_waitcnt lgkmcnt(0)"
+                     : "=s"(t[0]), "=s"(t[1]), "=s"(t[2]), "=s"(t[3]), "=s"(t[4]), "=s"(t[5]), "=s"(t[6]), "=s"(t[7]), "=s"(t[8]), "=s"(t[9]), "=s"(t[10]),
+                       "=s"(t[11]), "=s"(t[12]), "=s"(t[13]), "=s"(t[14]), "=s"(t[15])
+                     : "s"(p));
+    } else {
+        asm volatile(NCE_KA_LOAD(0) NCE_KA_LOAD(1) NCE_KA_LOAD(2) NCE_KA_LOAD(3) NCE_KA_LOAD(4) NCE_KA_LOAD(5) NCE_KA_LOAD(6) NCE_KA_LOAD(7) NCE_KA_LOAD(8)
+                     NCE_KA_LOAD(9) NCE_KA_LOAD(10) NCE_KA_LOAD(11) NCE_KA_LOAD(12) NCE_KA_LOAD(13) NCE_KA_LOAD(14) NCE_KA_LOAD(15) "s_waitcnt lgkmcnt(0)"
+                     : "=s"(t[0]), "=s"(t[1]), "=s"(t[2]), "=s"(t[3]), "=s"(t[4]), "=s"(t[5]), "=s"(t[6]), "=s"(t[7]), "=s"(t[8]), "=s"(t[9]), "=s"(t[10]),
+                       "=s"(t[11]), "=s"(t[12]), "=s"(t[13]), "=s"(t[14]), "=s"(t[15])
+                     : "s"(p));
+    }
+#undef NCE_KA_LOAD
+    __builtin_amdgcn_sched_barrier(0);  // (nothing that follows - in particular no argument load with its own wait - moves ahead of the requests)
+#endif
+}
+
 // Store 16 (or 8) consecutive channels of one pixel: one vector store when channels are compact, byte
 // stores at the channel stride for permuted output orders. p points at the first of those channels.
 __device__ __forceinline__ void store_channels16(uint8_t* p, int64_t sc, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {

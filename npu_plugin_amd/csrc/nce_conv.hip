@@ -25,6 +25,7 @@ constexpr int NTHREADS = 256;
 // PXF = 32-pixel fragments per wavefront; the workgroup tile is (4 * 32 * PXF) pixels x 64 channels.
 template <int PXF>
 __global__ __launch_bounds__(NTHREADS) void conv_igemm_kernel(ConvArgs a) {
+    prefetch_kernel_arguments<sizeof(ConvArgs)>();
     constexpr int BM = 128 * PXF;
     constexpr int NB = 2 * PXF;  // activation rows each thread stages per step
 

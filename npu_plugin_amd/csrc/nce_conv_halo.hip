@@ -26,6 +26,7 @@ constexpr int JMAX = 8;  // halo 16-byte loads per thread per input slice
 
 template <int WN, int WP, int AF, int BF, int KX>
 __global__ __launch_bounds__(64 * WN * WP) void conv_halo_kernel(ConvArgs a) {
+    prefetch_kernel_arguments<sizeof(ConvArgs)>();
     constexpr int NT = 64 * WN * WP;
     constexpr int BN = WN * AF * 32;
     constexpr int BM = WP * BF * 32;

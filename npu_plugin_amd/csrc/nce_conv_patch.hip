@@ -111,6 +111,7 @@ __device__ __forceinline__ int halo_piece(int key, int pos) {
 // epilogues or stand at a request, at 0.75 instead of 0.5 KiB of LDS reads per matrix instruction).
 template <int NF, int NPX, int ULOG, int NW>
 __global__ __launch_bounds__(64 * NW, NW / 4) void conv_patch_kernel(PatchArgs w) {
+    prefetch_kernel_arguments<sizeof(PatchArgs)>();
     constexpr int BN = 16 * NF;
     const ConvArgs& a = w.a;
 

@@ -56,6 +56,7 @@ constexpr int tiled_min_waves(int nwaves) {
 
 template <int WM, int WN, int TM, int TN, int NS, int KC, bool FZ>
 __global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_tiled_kernel(TiledArgs w) {
+    prefetch_kernel_arguments<sizeof(TiledArgs)>();
     constexpr int NW = WM * WN;
     constexpr int BM = 16 * TM * WM;
     constexpr int BN = 16 * TN * WN;

@@ -623,6 +623,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
 
 template <int NF, int BF, int MODE, int D, int LM>
 __global__ __launch_bounds__(512) void conv_wres_kernel(WresArgs w) {
+    prefetch_kernel_arguments<sizeof(WresArgs)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];  // [step][fragment][lane] x 16 bytes
     __shared__ WresSmemOf<NF, MODE> sm;
     const uint32_t group = xcd_tile(blockIdx.x, w.ngroups);
@@ -733,6 +734,7 @@ hipError_t launch_mode(WresArgs& w, int mode, int nwaves, int tpw, hipStream_t s
 // tap counters, row / column validity bits (any kernel up to 31 x 31). ASUM as in conv_wres_kernel.
 template <int NF, int BF, bool ASUM>
 __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
+    prefetch_kernel_arguments<sizeof(WresArgs)>();
     constexpr int OCT = 16 * NF;
     constexpr int BP = 16 * BF;
     constexpr int D = 4;
@@ -1203,6 +1205,7 @@ struct PkInputWait {
 };
 
 __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
+    prefetch_kernel_arguments<sizeof(PkArgs)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t sWt[];
     __shared__ __attribute__((aligned(16))) uint8_t sm_raw[sizeof(WresSmemOf<4, WRES_FAST>)];  // (the largest of the variants' tables)
     __shared__ uint32_t s_err;

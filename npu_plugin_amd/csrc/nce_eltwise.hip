@@ -43,6 +43,7 @@ typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 template <bool FLAT, int PATH, bool SIGNED>
 __global__ __launch_bounds__(256) void eltwise_kernel(EltArgs a) {
+    prefetch_kernel_arguments<sizeof(EltArgs)>();
     const TaskDev& t = a.t;
     const Box& box = a.box;
     const int32_t cgroups = box.bc >> 4;

@@ -83,6 +83,7 @@ struct WinArgs {
 // the general kernel pays three 64-bit divisions per item, which cost more than the window itself.
 template <int MODE, int KK, bool I32>
 __global__ __launch_bounds__(NT) void window_kernel(WinArgs a) {
+    prefetch_kernel_arguments<sizeof(WinArgs)>();
     // MODE_DW: [tap][SLAB_CH] floats of (w - zp_w); then per-channel FP64 scale constants
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ double sM[SLAB_CH], sB[SLAB_CH];
