@@ -74,6 +74,9 @@ struct WresArgs {
 #ifndef WRES_PART
 #define WRES_PART 0
 #endif
+#ifndef NCE_WB
+#define NCE_WB 4
+#endif
 hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream);
 #ifdef WRES_TRACE
 extern uint64_t* g_wres_trace;  // probe builds: 64 launch records, written round robin
@@ -397,7 +400,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         int32_t wpart[NF];  // sum of the (signed) weights this lane staged, per channel fragment
 #pragma unroll
         for (int f = 0; f < NF; ++f) wpart[f] = 0;
-        constexpr int WB = 4;       // weight loads in flight per lane while staging
+        constexpr int WB = NCE_WB;       // weight loads in flight per lane while staging
         constexpr int SB = WB / NF;  // steps per batch of loads
         uint4 v[SB][NF];
         // requests only (nothing here consumes a loaded value) ...
@@ -1225,6 +1228,16 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
         if (__builtin_amdgcn_readfirstlane(s_err) != 0) break;  // (uniform: read after a barrier)
         typedef const __attribute__((address_space(4))) PkLayer* table_ptr_t;
         const table_ptr_t L = (table_ptr_t)(uintptr_t)p.layers + (xcd * (uint32_t)p.nlayers + l);
+        // One word of every 64-byte line of the NEXT layer's table entry is requested now and consumed after this layer:
+        // the entry is then in the scalar cache when that layer starts (its fields are fetched where they are used, which
+        // from memory is a chain of cold misses at the head of every layer).
+        int32_t touch = 0;
+        if (l + 1 < p.nlayers) {
+            const __attribute__((address_space(4))) int32_t* const nl = reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(L + 1);
+#pragma unroll
+            for (int i = 0; i < (int)((sizeof(PkLayer) + 63) / 64); ++i) touch += nl[16 * i];
+        }
+        __builtin_amdgcn_sched_barrier(0);
         const int32_t variant = L->variant, nvirt = L->nvirt;
         const __attribute__((address_space(4))) WresArgs& w = L->w;
         const PkInputWait wait = {p.ctl, &s_err, deadline, l, xcd, target};
@@ -1244,6 +1257,7 @@ __global__ __launch_bounds__(512) void conv_wres_persistent_kernel(PkArgs p) {
         // This workgroup's share of layer l is stored: count it in. Every wave first waits until the L2 has acknowledged
         // all of its own stores (vmcnt(0), said explicitly: a workgroup-scope release need not wait for them), so that once
         // the barrier below has passed, the whole workgroup's output is in the XCD's L2 before thread 0 arrives.
+        asm volatile("" ::"s"(touch));       // (the words requested above are done with)
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters untouched
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
