@@ -493,7 +493,10 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
     // the FP64 product and sum are exact (24 x 25 significant bits).
     if (lane < OCT) {
         int32_t ws = 0;
-        for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
+        // (an input zero point equal to the storage offset - u8 around 128 - makes every weight-sum term zero: no need to
+        // collect the waves' partial sums then)
+        if (ASUM || a.da != 0)
+            for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
         // (with a weight zero-point offset dw the constant term S * 64 * da * dw joins; all below 2^30)
         const int32_t kdd = ASUM ? S * 64 * a.da * a.dw : 0;
         sCorr[wave][lane] = a.da * ws + kdd;
@@ -992,7 +995,10 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
     const EpiPack ep = epi_pack_setup(pu);
     if (lane < OCT) {
         int32_t ws = 0;
-        for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
+        // (an input zero point equal to the storage offset - u8 around 128 - makes every weight-sum term zero: no need to
+        // collect the waves' partial sums then)
+        if (ASUM || a.da != 0)
+            for (int i = 0; i < nwaves; ++i) ws += sWpart[i][lane];
         // (the host rejects reductions for which S * 64 * da * dw or dw * a pixel's sum could leave int32)
         const int32_t kdd = ASUM ? S * 64 * a.da * a.dw : 0;
         sCorr[wave][lane] = a.da * ws + kdd;
