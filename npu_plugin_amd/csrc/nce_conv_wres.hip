@@ -397,6 +397,8 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
             wrow_ok[f] = channel_of_frag_row<NF>(f, li) < noc;
             wrow[f] = wrow0 + (int64_t)(4 * f) * a.w_soc;
         }
+        // (an input zero point equal to the storage offset - u8 around 128 - makes every weight-sum term zero: no sums then)
+        const bool need_sums = ASUM || a.da != 0;  // uniform
         int32_t wpart[NF];  // sum of the (signed) weights this lane staged, per channel fragment
 #pragma unroll
         for (int f = 0; f < NF; ++f) wpart[f] = 0;
@@ -427,7 +429,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
 #pragma unroll
                     for (int f = 0; f < NF; ++f) {
                         const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
-                        wpart[f] += bytesum(sw);
+                        if (need_sums) wpart[f] += bytesum(sw);
                         *reinterpret_cast<uint4*>(sWt + ((size_t)st * NF + f) * 1024 + lane * 16) = sw;
                     }
                 }
@@ -451,7 +453,7 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         }
         // the four lanes of a row add up their pieces; the first of them publishes the wave's partial sum
 #pragma unroll
-        for (int f = 0; f < NF; ++f) {
+        for (int f = 0; need_sums && f < NF; ++f) {
             int32_t p = wpart[f];
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
