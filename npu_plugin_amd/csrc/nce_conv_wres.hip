@@ -875,7 +875,7 @@ __global__ __launch_bounds__(512) void conv_wres_chunked_kernel(WresArgs w) {
 #pragma unroll
                 for (int f = 0; f < NF; ++f) {
                     const uint4 sw = make_uint4(v[j][f].x ^ a.w_xor, v[j][f].y ^ a.w_xor, v[j][f].z ^ a.w_xor, v[j][f].w ^ a.w_xor);
-                    wpart[f] += bytesum(sw);
+                    if (ASUM || a.da != 0) wpart[f] += bytesum(sw);  // (uniform: no sums when the input zero-point term is zero)
                     *reinterpret_cast<uint4*>(sWt + ((size_t)(st - sbase) * NF + f) * 1024 + lane * 16) = sw;
                 }
             }
