@@ -49,13 +49,14 @@ using namespace lds_detail;  // swz (bank-conflict-free piece placement), vmcnt_
 
 // Waves per SIMD the register budget must allow (vector + accumulation registers share 512 per lane and SIMD): two
 // workgroups of four waves, or one of eight, per CU at the least - a lone wave per SIMD leaves every LDS and barrier
-// round trip of the step loop exposed.
-constexpr int tiled_min_waves(int nwaves) {
-    return nwaves >= 8 ? 2 : 2;
+// round trip of the step loop exposed. Eight waves of 32 x 64 outputs (eight accumulator fragments) fit 128 registers: two
+// such workgroups share a CU, four waves per SIMD.
+constexpr int tiled_min_waves(int nwaves, int frags) {
+    return nwaves >= 8 && frags <= 8 ? 4 : 2;
 }
 
 template <int WM, int WN, int TM, int TN, int NS, int KC, bool FZ>
-__global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN)) void conv_tiled_kernel(TiledArgs w) {
+__global__ __launch_bounds__(64 * WM * WN, tiled_min_waves(WM * WN, TM * TN)) void conv_tiled_kernel(TiledArgs w) {
     prefetch_kernel_arguments<sizeof(TiledArgs)>();
     constexpr int NW = WM * WN;
     constexpr int BM = 16 * TM * WM;
@@ -365,8 +366,8 @@ hipError_t launch_shape(TiledArgs& w, bool fused, hipStream_t stream) {
 }  // namespace
 
 // Shapes: 1 = 128 px x 128 ch (4 waves), 2 = 64 px x 128 ch (4 waves), 3 = 256 px x 128 ch (8 waves),
-// 4 = 128 px x 64 ch (4 waves), 5 = shape 1 with steps of 128 bytes of the reduction (input channels a multiple of 128).
-// shape 0 = automatic.
+// 4 = 128 px x 64 ch (4 waves), 5 = shape 1 with steps of 128 bytes of the reduction (input channels a multiple of 128),
+// 6 = shape 5 as eight waves of 32 px x 64 ch, two workgroups = sixteen waves per CU. shape 0 = automatic.
 hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, const FuseAdd* fuse) {
     if (a.IC % 64 != 0 || a.dw != 0 || a.KY > 32 || a.KX > 32) return hipErrorNotSupported;
     if (a.M > 0x7fffffff - 1024) return hipErrorNotSupported;
@@ -385,7 +386,7 @@ hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, c
     if (shape == 0) {
         // The largest tile that still gives every CU about two workgroups.
         const auto groups = [&](int bm, int bn) { return (((int64_t)a.M + bm - 1) / bm) * ((a.bc + bn - 1) / bn); };
-        shape = groups(128, 128) >= 512 ? (a.IC % 128 == 0 ? 5 : 1) : 2;
+        shape = groups(128, 128) >= 512 ? (a.IC % 128 == 0 ? 6 : 1) : 2;
     }
     const bool fz = fuse != nullptr;
     switch (shape) {
@@ -394,6 +395,7 @@ hipError_t launch_conv_tiled(const ConvArgs& a, hipStream_t stream, int shape, c
     case 3: return launch_shape<4, 2, 4, 4, 3>(w, fz, stream);
     case 4: return launch_shape<2, 2, 4, 2, 4>(w, fz, stream);
     case 5: return launch_shape<2, 2, 4, 4, 2, 2>(w, fz, stream);
+    case 6: return launch_shape<4, 2, 2, 4, 2, 2>(w, fz, stream);
     default: return hipErrorNotSupported;
     }
 }

@@ -28,7 +28,7 @@ TILED_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("shape", TILED_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}x{s[2]}x{s[3]}_{s[4]}_k{s[5][0]}s{s[6][0]}")
 def test_conv_tiled_shapes(tuned, shape, tile):
     n, h, w, ic, oc, k, s, pads, in_zp = shape
@@ -37,7 +37,7 @@ def test_conv_tiled_shapes(tuned, shape, tile):
                       ppe=dict(mode=nce.PPE_LPRELU, clamp_low=0, clamp_high=250, lrelu_mult=1638, lrelu_shift=14)), executor)
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6])
 def test_conv_tiled_types_and_modes(tuned, tile):
     executor = tuned(NCE_HIP_CONV_TILED=tile)
     wide = dict(k=(3, 3), pads=(1, 1, 1, 1))
@@ -57,7 +57,7 @@ def test_conv_tiled_types_and_modes(tuned, tile):
     check(K.conv_case(1435, 2, 11, 11, 48, 64, in_zp=131, **wide), executor)
 
 
-@pytest.mark.parametrize("tile", [1, 2, 4, 5])
+@pytest.mark.parametrize("tile", [1, 2, 4, 5, 6])
 def test_conv_tiled_variants_and_output_orders(tuned, tile):
     executor = tuned(NCE_HIP_CONV_TILED=tile)
     full = K.conv_case(1305, 2, 24, 20, 128, 192)
@@ -76,7 +76,7 @@ def test_conv_tiled_variants_and_output_orders(tuned, tile):
 
 
 @pytest.mark.parametrize("conv_first,in_place", [(True, False), (False, True)])
-@pytest.mark.parametrize("tile", [1, 2, 3, 5])
+@pytest.mark.parametrize("tile", [1, 2, 3, 5, 6])
 def test_conv_tiled_with_fused_residual_add(tuned, conv_first, in_place, tile):
     for ic, oc, out_signed, out_zp in ((64, 256, False, 128), (128, 80, True, -3), (512, 144, False, 7)):
         lo, hi = (-128, 127) if out_signed else (0, 255)
