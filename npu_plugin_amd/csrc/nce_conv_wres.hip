@@ -74,8 +74,15 @@ struct WresArgs {
 #ifndef WRES_PART
 #define WRES_PART 0
 #endif
+// Weight loads a lane keeps in flight while a slice is staged. Eight for the persistent form, whose layers stage while other
+// workgroups of the XCD still compute (measured on the ResNet-50 graph at batch 32: 639 against 648 us); for separate launches
+// eight is level with four (-0.4 % at batch 32 and 64, +1.4 % at batch 8) and sixteen slower (+2 %: registers).
 #ifndef NCE_WB
+#if WRES_PART == 3
+#define NCE_WB 8
+#else
 #define NCE_WB 4
+#endif
 #endif
 hipError_t launch_wres_nf4(WresArgs& w, int bf, int mode, int nwaves, int tpw, hipStream_t stream);
 #ifdef WRES_TRACE
