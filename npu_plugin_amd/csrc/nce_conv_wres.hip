@@ -348,10 +348,10 @@ __device__ __forceinline__ void conv_wres_body(const WArgs& w, const uint32_t gr
         for (int j = 0; j < D; ++j) load_b(fb[j], from_table);
     };
     // ---- stage the channel slice's weights in operand order; per-channel constants ---------------
-    // The slice is S * NF operand fragments of 1 KiB: (step, channel fragment) -> 16 rows x 64 bytes. A wave
-    // fetches a fragment with lane 4i + k on 16-byte piece k of row i (a row's 64 bytes from four neighbouring
-    // lanes), permutes the registers into operand order (lane 16k + i) and writes the fragment with one
-    // linear, bank-conflict-free store.
+    // The slice is S * NF blocks of 1 KiB: (step, channel fragment) -> 16 rows x 64 bytes, kept row-major with the four
+    // 16-byte pieces of a row permuted (nce_conv_lds.h). A wave fetches a block with the four lanes 4i .. 4i + 3 on the
+    // pieces of row i (a row's 64 bytes from four neighbouring lanes, each lane on the piece that belongs at ITS position)
+    // and writes it where it stands: one linear, bank-conflict-free store, no lane exchange.
     {
         const int li = lane >> 2;
         const int64_t acc_bound = min((int64_t)a.ktot * 65025, (int64_t)2147483648LL);
