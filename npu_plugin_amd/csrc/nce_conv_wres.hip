@@ -1,8 +1,8 @@
 // CONV task, weights-resident implicit GEMM on v_mfma_i32_16x16x64_i8.
 //
 // A workgroup owns one slice of 16*NF output channels and a run of pixel tiles. It stages the WHOLE
-// reduction (KY*KX*IC bytes) of its channels in LDS once, already in MFMA operand order, and after that
-// single barrier its wavefronts never synchronise again: each wave walks its own tiles of 16*BF output
+// reduction (KY*KX*IC bytes) of its channels in LDS once, as 1 KiB blocks that one ds_read_b128 per lane turns
+// into an MFMA operand, and after that single barrier its wavefronts never synchronise again: each wave walks its own tiles of 16*BF output
 // pixels, loads the activation operand straight from global memory and runs the fused PPE on its
 // accumulators.
 //
@@ -13,9 +13,11 @@
 //
 // Lane order of memory instructions matters more than the bytes they move: a global load whose four
 // neighbouring lanes read one 64-byte run costs the texture addresser a quarter of one whose runs are
-// spread over four quads of lanes, and an LDS store whose lanes share a bank is serialised. Hence the
-// weights (always) and the activations (template flag TRL, when pixels are more than 64 bytes apart) are
-// fetched with lane 4*row + piece and moved into operand order (lane 16*piece + row) with ds_bpermute_b32.
+// spread over four quads of lanes, and an LDS access whose lanes share a bank group is serialised. Hence both
+// operands are fetched with lane 4*row + piece: the weights are stored to LDS as fetched (row-major blocks whose
+// pieces are permuted so that the operand reads are conflict-free, nce_conv_lds.h), the activations (template flag
+// TRL, when pixels are more than 64 bytes apart) are moved into operand order (lane 16*piece + row) with
+// ds_bpermute_b32.
 //
 // The reduction is cut in steps of 64 bytes = four 16-byte units; unit u covers bytes 16u..16u+15 of
 // the OYXI weight row, i.e. tap u / (IC/16), input channels 16 * (u % (IC/16)). With IC a multiple of
