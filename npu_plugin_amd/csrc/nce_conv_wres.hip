@@ -1147,7 +1147,9 @@ hipError_t launch_conv_wres(const ConvArgs& a, hipStream_t stream, bool allow_ch
     // (per-XCD form: an eighth of the work on an eighth of the CUs - the same choices as for the whole task)
     const int cus = tls_launch.per_xcd ? 32 : 256;
     const int64_t want = ((w.ntaps == 1 && w.nsteps > 1) ? 6000 : 1500) * cus / 256;
-    int nf = nf4_ok ? 4 : 2, bf = 4;
+    // (per-XCD form: tiles of at most 32 pixels - the persistent kernel carries no 64-pixel instantiation, whose registers
+    // every layer's path would pay for)
+    int nf = nf4_ok ? 4 : 2, bf = tls_launch.per_xcd ? 2 : 4;
     while (bf > 1 && wave_tiles(nf, bf) < want) bf >>= 1;
     if (nf == 4 && wave_tiles(nf, bf) < 1500 * cus / 256) nf = 2;
     const int nwaves = 8;
@@ -1187,7 +1189,8 @@ namespace {
     X(4, 2, 1, WRES_FAST_MASK, 4, LM_TRL) X(5, 4, 2, WRES_FAST_MASK, 3, LM_TRL)  \
     X(6, 4, 2, WRES_FAST, 2, LM_PLAIN_FZ) X(8, 2, 1, WRES_FAST, 4, LM_TRL)      \
     X(10, 4, 2, WRES_FAST, 4, LM_PLAIN_FZ) X(11, 4, 2, WRES_FAST, 4, LM_PLAIN)     \
-    X(12, 4, 2, WRES_FAST, 2, LM_PLAIN)
+    X(12, 4, 2, WRES_FAST, 2, LM_PLAIN) X(13, 4, 2, WRES_FAST, 1, LM_PLAIN) X(14, 4, 2, WRES_FAST, 1, LM_PLAIN_FZ)          \
+    X(15, 4, 2, WRES_FAST_MASK, 3, LM_TBL)
 
 // Device table: [xcd][layer], the launch arguments of that XCD's share (pointers already advanced to its images).
 struct PkLayer {
